@@ -31,12 +31,20 @@ class CacheGroup:
     window: Optional[int]          # None: no window
     runs: Tuple[int, ...]          # entries of the model's order that keep their cache here
     chunk: Optional[int] = None    # None: no chunks; else a query reads keys of its own chunk of positions only
+    keep_first: int = 0            # positions at a sequence's start that every query reads, whatever the window
 
     @property
     def reach(self) -> Optional[int]:
-        """How many positions back a query can read at most (itself included); None: all of them."""
+        """How many positions back a query can read at most (itself included), the kept first positions
+        aside; None: all of them."""
         bounds = [b for b in (self.window, self.chunk) if b is not None]
         return min(bounds) if bounds else None
+
+    def kept_pages(self, page_size: int) -> int:
+        """The leading pages that hold kept first positions: they stay with the request until it ends."""
+        if self.reach is None or self.keep_first <= 0:
+            return 0
+        return (self.keep_first + page_size - 1) // page_size
 
     def first_key(self, query: int) -> int:
         """The first position that a query at position `query` reads."""
@@ -61,7 +69,7 @@ def plan_groups(needs) -> Tuple[List[CacheGroup], List[int]]:
     """From the per-run needs (PagedKV / FixedState / None) the page groups, and the runs
     that keep fixed state.  A need is recognised by its attributes, so that this module
     imports nothing from the parts."""
-    by_reach: Dict[Tuple[Optional[int], Optional[int]], List[int]] = {}
+    by_reach: Dict[Tuple[Optional[int], Optional[int], int], List[int]] = {}
     state_runs: List[int] = []
     for i, need in enumerate(needs):
         if need is None:
@@ -70,12 +78,13 @@ def plan_groups(needs) -> Tuple[List[CacheGroup], List[int]]:
             if hasattr(part, "tensors"):
                 state_runs.append(i)
             elif hasattr(part, "num_kv_heads"):
-                by_reach.setdefault((part.window, getattr(part, "chunk", None)), []).append(i)
+                keep = int(getattr(part, "keep_first", 0) or 0) if part.window is not None else 0
+                by_reach.setdefault((part.window, getattr(part, "chunk", None), keep), []).append(i)
             else:
                 raise ValueError(f"run {i}: unknown cache need {part!r}")
     # the all-keys group first, then by window and chunk
-    keys = sorted(by_reach, key=lambda wc: (wc != (None, None), wc[0] or 0, wc[1] or 0))
-    return [CacheGroup(w, tuple(by_reach[(w, c)]), c) for w, c in keys], state_runs
+    keys = sorted(by_reach, key=lambda wc: (wc[:2] != (None, None), wc[0] or 0, wc[1] or 0, wc[2]))
+    return [CacheGroup(w, tuple(by_reach[(w, c, kf)]), c, kf) for w, c, kf in keys], state_runs
 
 
 def chain_hash(tokens: Sequence[int], prefix: int = -1) -> int:
@@ -149,8 +158,10 @@ class CacheManager:
         first_query = rc.num_tokens if first_query is None else first_query
         out = []
         for g, table in enumerate(rc.tables):
+            want = self._wanted_pages(g, new_len, step_end)
             lo = max(len(table), self._first_needed_page(g, first_query))
-            out.append(max(0, self._wanted_pages(g, new_len, step_end) - lo))
+            kept = min(self.groups[g].kept_pages(self.page_size), lo, want)      # kept first pages not yet in the table
+            out.append(max(0, want - lo) + max(0, kept - len(table)))
         return out
 
     def peak_pages(self, num_tokens: int, portion: int) -> List[int]:
@@ -164,7 +175,7 @@ class CacheManager:
                 out.append(total)
             else:
                 span = group.reach - 1 + max(1, min(portion, num_tokens))       # positions a step touches, at any offset
-                out.append(min(total, (span + self.page_size - 2) // self.page_size + 1))
+                out.append(min(total, (span + self.page_size - 2) // self.page_size + 1 + group.kept_pages(self.page_size)))
         return out
 
     def can_reserve(self, request: Hashable, new_len: int, first_query: Optional[int] = None,
@@ -196,7 +207,8 @@ class CacheManager:
         out = []
         for g, table in enumerate(rc.tables):
             upto = min(self._first_needed_page(g, first_query), len(table))
-            out.append(sum(1 for p in table[:upto] if p >= 0 and self.pools[g].ref_count[p] == 1))
+            kept = self.groups[g].kept_pages(self.page_size)
+            out.append(sum(1 for p in table[kept:upto] if p >= 0 and self.pools[g].ref_count[p] == 1))
         return out
 
     def reserve(self, request: Hashable, new_len: int, first_query: Optional[int] = None,
@@ -212,12 +224,13 @@ class CacheManager:
         for g, (pool, table) in enumerate(zip(self.pools, rc.tables)):
             want = self._wanted_pages(g, new_len, step_end)
             first_page = self._first_needed_page(g, first_query)
-            for i in range(min(first_page, len(table))):
+            kept = self.groups[g].kept_pages(self.page_size)
+            for i in range(kept, min(first_page, len(table))):
                 if table[i] >= 0:
                     pool.give_back(table[i])
                     table[i] = -1
             while len(table) < want:
-                table.append(pool.take() if len(table) >= first_page else -1)
+                table.append(pool.take() if len(table) >= first_page or len(table) < kept else -1)
         if step_end is not None and any(group.reach is not None for group in self.groups):
             new_len = min(new_len, step_end)                    # positions that every group covers
         rc.num_tokens = max(rc.num_tokens, new_len)
@@ -248,12 +261,14 @@ class CacheManager:
             for g, p in enumerate(pages):
                 found[g].append(p)
         hits = 0
+        kept = [group.kept_pages(ps) for group in self.groups]
         for n in range(len(found[0]), 0, -1):
-            if all(-1 not in found[g][self._first_needed_page(g, n * ps):n] for g in range(len(self.groups))):
+            if all(-1 not in found[g][self._first_needed_page(g, n * ps):n] and -1 not in found[g][:min(kept[g], n)]
+                   for g in range(len(self.groups))):
                 hits = n
                 break
-        return hits, [[p if i >= self._first_needed_page(g, hits * ps) else -1 for i, p in enumerate(found[g][:hits])]
-                      for g in range(len(self.groups))]
+        return hits, [[p if i >= self._first_needed_page(g, hits * ps) or i < kept[g] else -1
+                       for i, p in enumerate(found[g][:hits])] for g in range(len(self.groups))]
 
     def can_admit(self, tokens: Sequence[int], first_step: Optional[int] = None) -> int:
         """-1 if the pages for all of `tokens` are not free, else the number of leading pages

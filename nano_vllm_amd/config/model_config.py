@@ -504,3 +504,186 @@ class MafaraxConfig:
         if self.eos_token_id is not None:
             out["eos_token_id"] = list(self.eos_token_id)
         return out
+
+
+# ---------------------------------------------------------------------------- Kirisun
+def _count(d: Mapping[str, Any], key: str, where: str, default=None) -> int:
+    """A whole number that may be zero."""
+    v = d.get(key, default)
+    if v is None or isinstance(v, bool) or not isinstance(v, (int, float)) or v != int(v) or int(v) < 0:
+        raise ConfigError(f"{where}: key {key!r} must be a whole number, zero or more, got {v!r}")
+    return int(v)
+
+
+@dataclass(frozen=True)
+class GatedAttentionConfig:
+    """Grouped attention with normed query and key heads, a rotation of the first rot_dims channels of a head
+    (every frequency divided by rot_factor; rot_dims 0: none), scores scale * q.k capped smoothly at +-softcap
+    (None: no cap), a window of `window` positions that also keeps the first keep_first positions of the
+    sequence in sight (window None: every earlier position), a sink of score 0 in the softmax, and an
+    output gate."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    softcap: Optional[float] = None
+    window: Optional[int] = None
+    keep_first: int = 0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_factor: float = 1.0
+
+
+@dataclass(frozen=True)
+class ChannelDeltaConfig:
+    """The delta-rule mixer with a decay per key channel: `heads` value heads of vdim, kv_heads query/key heads
+    of dim, short convolutions of `conv` taps; the ranks of the two-step projections of the decay and of the
+    output gate are read from the tensors' shapes unless the mixer names them (decay_rank, gate_rank: what a
+    folder of random weights is drawn with)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+    decay_rank: Optional[int] = None
+    gate_rank: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class SoftmaxExpertsConfig:
+    """A routed feed-forward of gated experts: `top` of `experts` experts of inner size ff, weighted by the
+    softmax over the chosen router logits."""
+    experts: int
+    top: int
+    ff: int
+
+
+@dataclass(frozen=True)
+class KirisunLayer:
+    kind: str                                    # "attention" | "channel_delta"
+    mixer: Any                                   # GatedAttentionConfig | ChannelDeltaConfig
+    mlp: Optional[SoftmaxExpertsConfig]
+
+
+@dataclass(frozen=True)
+class KirisunConfig:
+    """Kirisun: layers with a norm before and after each sublayer on a float32 residual stream that takes each
+    sublayer's normed output times residual_mult; the mixer is, layer by layer, a gated window attention or
+    the channel-wise delta rule; the feed-forward a mixture of gated experts, or absent; the embedding is
+    multiplied by embedding_scale.  config.json gives every size and constant, layer by layer."""
+    vocab: int
+    width: int
+    eps: float
+    residual_mult: float
+    embedding_scale: float
+    layers: Tuple[KirisunLayer, ...]
+    dtype: str = "bfloat16"
+    eos_token_id: Optional[Tuple[int, ...]] = None
+    architecture: str = "Kirisun"
+
+    @classmethod
+    def from_dict(cls, d: Mapping[str, Any]) -> "KirisunConfig":
+        where = "config.json"
+        entries = d.get("layers")
+        if not isinstance(entries, (list, tuple)) or not entries:
+            raise ConfigError(f"{where}: key 'layers' must be a list of layers")
+        layers = []
+        for i, entry in enumerate(entries):
+            at = f"{where}: layers[{i}]"
+            if not isinstance(entry, Mapping):
+                raise ConfigError(f"{at} must be an object")
+            kind = entry.get("type")
+            m = _section(entry, "mixer", at)
+            ma = at + ".mixer"
+            sizes = dict(heads=_whole(m, "heads", ma), kv_heads=_whole(m, "kv_heads", ma), dim=_whole(m, "dim", ma),
+                         vdim=_whole(m, "vdim", ma))
+            if kind == "attention":
+                rot, mask = m.get("rot"), m.get("mask")
+                dims, base, factor = 0, 10000.0, 1.0
+                if rot is not None:
+                    dims = _whole(rot, "dims", ma + ".rot")
+                    base = _require(rot, "base", float, ma + ".rot")
+                    if rot.get("scaling") is not None:
+                        factor = _require(rot["scaling"], "factor", float, ma + ".rot.scaling")
+                cap = m.get("softcap")
+                mixer = GatedAttentionConfig(
+                    **sizes, scale=_require(m, "scale", float, ma),
+                    softcap=None if cap is None else _require(m, "softcap", float, ma),
+                    window=None if mask is None else _whole(mask, "size", ma + ".mask"),
+                    keep_first=0 if mask is None else _count(mask, "keep_first", ma + ".mask", 0),
+                    rot_dims=dims, rot_base=base, rot_factor=factor)
+            elif kind == "channel_delta":
+                mixer = ChannelDeltaConfig(**sizes, conv=_whole(m, "conv", ma),
+                                           decay_rank=None if m.get("decay_rank") is None else _whole(m, "decay_rank", ma),
+                                           gate_rank=None if m.get("gate_rank") is None else _whole(m, "gate_rank", ma))
+            else:
+                raise ConfigError(f"{at}: type must be 'attention' or 'channel_delta', got {kind!r}")
+            mlp = entry.get("mlp")
+            experts = None
+            if mlp is not None:
+                fa = at + ".mlp"
+                if not isinstance(mlp, Mapping) or mlp.get("kind", "moe") != "moe":
+                    raise ConfigError(f"{fa} must be null or an object of kind 'moe', got {mlp!r}")
+                router = _section(mlp, "router", fa)
+                experts = SoftmaxExpertsConfig(experts=_whole(router, "experts", fa + ".router"),
+                                               top=_whole(router, "top", fa + ".router"),
+                                               ff=_whole(_section(mlp, "expert", fa), "ff", fa + ".expert"))
+            layers.append(KirisunLayer(kind, mixer, experts))
+        norm = _section(d, "norm", where)
+        embedding = d.get("embedding") or {}
+        eos = d.get("eos_token_id")
+        eos = (eos,) if isinstance(eos, int) else tuple(int(x) for x in eos) if isinstance(eos, (list, tuple)) else None
+        cfg = cls(vocab=_whole(d, "vocab", where), width=_whole(d, "width", where),
+                  eps=_require(norm, "eps", float, where + ": norm"),
+                  residual_mult=float(d["residual_mult"]) if d.get("residual_mult") is not None else 1.0,
+                  embedding_scale=float(embedding["scale"]) if embedding.get("scale") is not None else 1.0,
+                  layers=tuple(layers), dtype=canonical_dtype(d.get("dtype") or d.get("torch_dtype") or "bfloat16"),
+                  eos_token_id=eos, architecture=d.get("architecture") or (d.get("architectures") or ["Kirisun"])[0])
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if not (self.eps > 0):
+            raise ConfigError(f"config.json: norm.eps must be positive, got {self.eps}")
+        for i, layer in enumerate(self.layers):
+            at = f"config.json: layers[{i}]"
+            m, f = layer.mixer, layer.mlp
+            if m.heads % m.kv_heads:
+                raise ConfigError(f"{at}: {m.heads} heads do not divide into {m.kv_heads} kv_heads")
+            if layer.kind == "attention":
+                if m.rot_dims % 2 or m.rot_dims > m.dim or (m.rot_dims and not (m.rot_base > 0 and m.rot_factor > 0)):
+                    raise ConfigError(f"{at}: rot.dims {m.rot_dims} must be even and at most dim {m.dim}, rot.base and "
+                                      f"the scaling factor positive")
+                if not (m.scale > 0) or (m.softcap is not None and not (m.softcap > 0)):
+                    raise ConfigError(f"{at}: scale and softcap must be positive, got {m.scale} and {m.softcap}")
+            if f is not None and f.top > f.experts:
+                raise ConfigError(f"{at}: {f.top} experts a token out of {f.experts}")
+
+    def to_dict(self) -> dict:
+        """The config.json that describes this configuration."""
+        entries = []
+        for layer in self.layers:
+            m, f = layer.mixer, layer.mlp
+            mixer = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim, "vdim": m.vdim}
+            if layer.kind == "attention":
+                mixer["scale"] = m.scale
+                if m.softcap is not None:
+                    mixer["softcap"] = m.softcap
+                if m.window is not None:
+                    mixer["mask"] = {"size": m.window, "keep_first": m.keep_first}
+                if m.rot_dims:
+                    mixer["rot"] = {"dims": m.rot_dims, "base": m.rot_base, "scaling": {"factor": m.rot_factor}}
+            else:
+                mixer["conv"] = m.conv
+                for key in ("decay_rank", "gate_rank"):
+                    if getattr(m, key) is not None:
+                        mixer[key] = getattr(m, key)
+            mlp = None if f is None else {"kind": "moe", "expert": {"ff": f.ff}, "router": {"experts": f.experts, "top": f.top}}
+            entries.append({"type": layer.kind, "mixer": mixer, "mlp": mlp})
+        out = {"architecture": self.architecture, "vocab": self.vocab, "width": self.width, "norm": {"eps": self.eps},
+               "residual_mult": self.residual_mult, "embedding": {"scale": self.embedding_scale}, "layers": entries,
+               "torch_dtype": self.dtype}
+        if self.eos_token_id is not None:
+            out["eos_token_id"] = list(self.eos_token_id)
+        return out

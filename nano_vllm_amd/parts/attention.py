@@ -19,6 +19,13 @@ Options beyond the reference's attention, each a parameter:
                                     chunk ... p only: the sequence is cut into chunks counted from its
                                     position 0, wherever a prompt was cut for processing
     o_bias                          a bias on the output projection
+    softcap                         scores capped smoothly: s <- softcap * tanh(s / softcap), after the scale
+    keep_first (with a window)      every query also reads the first keep_first positions of its sequence,
+                                    however far back they lie; they keep their own positions
+    sink_value                      a sink that is a constant (0: the softmax's denominator gains 1), no tensor
+    gate "sigmoid"                  the heads' outputs are multiplied, entry by entry, with sigmoid(x Wg^T)
+                                    before the output projection; Wg [heads * v_head_dim, hidden] is packed
+                                    below q, k and v into the one projection
 With values of their own size (or whole-projection norms, or a temperature) the position encoding's
 rotation is applied by the same preparation kernel, from the cosines and sines of the step's tokens
 (position_encoding.step_table): such a model needs no table of all positions.
@@ -32,6 +39,8 @@ from __future__ import annotations
 
 from typing import Dict, Mapping
 
+import torch
+
 from .base import BuildContext, ParamDecl, Part, Source
 from .registry import register_part
 from .spec import PagedKV
@@ -44,7 +53,9 @@ class Attention(Part):
     projects q only and reads another run's keys and values), v_head_dim (None: head_dim),
     qk_norm_scope ("head" | "projection"), q_temperature (None or {"coef", "every"}), sink (bool),
     chunk (None or positions), o_bias (bool), step_rotation (bool: rotate from the step's own table
-    also where the per-head kernel could serve), and the names of the checkpoint tensors (q_name, ..., q_norm_name, k_norm_name, sink_name)."""
+    also where the per-head kernel could serve), softcap (None or a positive number), keep_first (positions),
+    sink_value (None or a number), gate (None or "sigmoid"), and the names of the checkpoint tensors (q_name, ...,
+    q_norm_name, k_norm_name, sink_name, g_name)."""
 
     def __init__(self, params: Mapping, build: BuildContext):
         super().__init__(params, build)
@@ -82,15 +93,32 @@ class Attention(Part):
         self.temp_coef = float(temp["coef"]) if temp else 0.0
         self.temp_every = int(temp["every"]) if temp else 1
         self.sink = bool(p.get("sink", False))
+        sink_value = p.get("sink_value")
+        self.sink_value = None if sink_value is None else float(sink_value)
+        if self.sink and self.sink_value is not None:
+            raise ValueError("attention: a learned sink and a constant one exclude each other")
+        cap = p.get("softcap")
+        self.softcap = None if cap is None else float(cap)
+        if self.softcap is not None and not self.softcap > 0:
+            raise ValueError(f"attention: a softcap of {self.softcap}")
+        self.keep_first = int(p.get("keep_first") or 0) if self.window is not None else 0
+        if self.keep_first < 0:
+            raise ValueError(f"attention: keep_first {self.keep_first}")
+        self.gate = p.get("gate")
+        if self.gate not in (None, "sigmoid"):
+            raise ValueError(f"attention: gate must be 'sigmoid' or absent, got {self.gate!r}")
+        self.g_name = p.get("g_name", "g_proj")
+        self._device = build.device
+        self._sink_tensor = None
         # The whole-projection preparation has its own kernel, which also scales q by its temperature
         # and stores values of their own size; the per-head one rotates.  Each does what its model needs.
         self.row_prepare = self.norm_scope == "projection" or self.temp_coef != 0.0 or self.v_head_dim != self.head_dim \
-            or bool(p.get("step_rotation", False))
+            or bool(p.get("step_rotation", False)) or self.gate is not None
         if self.row_prepare and self.position_encoding is not None and not hasattr(self.position_encoding, "step_table"):
             raise ValueError("attention: with whole-projection norms, a query temperature or values of their own "
                              "size the position encoding must offer step_table")
-        if self.row_prepare and self.qk_norm and self.norm_scope == "head":
-            raise ValueError("attention: per-head norms go with equal head sizes and no query temperature")
+        if self.gate is not None and (self.shared or self.bias):
+            raise ValueError("attention: an output gate goes with a cache of the run's own and no biases")
 
     @property
     def kernel_modules(self):
@@ -111,6 +139,9 @@ class Attention(Part):
         else:
             shards = ((self.q_name, 0, q), (self.k_name, q, kv), (self.v_name, q + kv, vv))
             rows = q + kv + vv
+            if self.gate is not None:
+                shards += ((self.g_name, rows, self.heads * self.v_head_dim),)
+                rows += self.heads * self.v_head_dim
         d["qkv_proj.weight"] = ParamDecl((rows, h), sources=tuple(Source(f"{n}.weight", r, c) for n, r, c in shards))
         if self.bias:
             d["qkv_proj.bias"] = ParamDecl((rows,), sources=tuple(Source(f"{n}.bias", r, c) for n, r, c in shards))
@@ -134,7 +165,16 @@ class Attention(Part):
             return None
         return PagedKV(self.kv_heads, self.head_dim, self.window,
                        None if self.v_head_dim == self.head_dim else self.v_head_dim,
-                       None if self.chunk is None else int(self.chunk))
+                       None if self.chunk is None else int(self.chunk), self.keep_first)
+
+    def _sinks(self):
+        if self.sink:
+            return self.weights.get("sinks")
+        if self.sink_value is None:
+            return None
+        if self._sink_tensor is None:          # made on first use: building a part touches no device
+            self._sink_tensor = torch.full((self.heads,), self.sink_value, dtype=torch.float32, device=self._device)
+        return self._sink_tensor
 
     # ------------------------------------------------------------------ forward
     def forward(self, x, batch, cache):
@@ -144,8 +184,13 @@ class Attention(Part):
         # deferred: the products below are handed to the q/k preparation and to the block's norm only
         pe = self.position_encoding
         table = pe.rotary_table() if pe is not None and not self.row_prepare else None
+        # (with a gate the row also holds the gate's columns, which outlive the preparation: a tensor, not partial sums)
         qkv = k.linear(x, w["qkv_proj.weight"], w.get("qkv_proj.bias"),
-                       deferred=self.row_prepare or pe is None or table is not None)
+                       deferred=self.gate is None and (self.row_prepare or pe is None or table is not None))
+        gate = None
+        if self.gate is not None:
+            qkv_width = (self.heads + self.kv_heads) * self.head_dim + self.kv_heads * self.v_head_dim
+            gate, qkv = qkv[:, qkv_width:], qkv[:, :qkv_width]
         group = batch.groups[cache.group]
         slots = None if self.shared else group.slot_mapping
         kc, vc = (None, None) if self.shared else (cache.k, cache.v)
@@ -153,6 +198,8 @@ class Attention(Part):
         kw = w.get("k_norm.weight")
         if self.row_prepare:
             extra = {"rot_table": pe.step_table(batch)} if pe is not None else {}
+            if self.qk_norm and self.norm_scope == "head":
+                extra["norm_per_head"] = True
             q = k.qk_rownorm_store(qkv, self.heads, kv_heads, self.head_dim, self.v_head_dim, qw, kw, self.eps,
                                    batch.positions, self.temp_coef, self.temp_every, slots, kc, vc, **extra)
         elif pe is None or table is not None:
@@ -169,12 +216,19 @@ class Attention(Part):
                 k.qk_norm_rope_store(qkv, self.heads, kv_heads, self.head_dim, None, None, self.eps, None, None,
                                      slots, kc, vc)
         extra = {"chunk": int(self.chunk)} if self.chunk is not None else {}
-        if self.sink or self.v_head_dim != self.head_dim:
+        if self.softcap is not None:
+            extra["softcap"] = self.softcap
+        if self.keep_first:
+            extra["keep_first"] = self.keep_first
+        sinks = self._sinks()
+        if sinks is not None or self.v_head_dim != self.head_dim:
             o = k.paged_attention(q, self.heads, self.kv_heads, self.head_dim, cache.k, cache.v, batch, cache.group,
-                                  self.scale, self.window, v_head_dim=self.v_head_dim, sinks=w.get("sinks"), **extra)
+                                  self.scale, self.window, v_head_dim=self.v_head_dim, sinks=sinks, **extra)
         else:
             o = k.paged_attention(q, self.heads, self.kv_heads, self.head_dim, cache.k, cache.v, batch, cache.group,
                                   self.scale, self.window, **extra)
+        if gate is not None:
+            o = k.sigmoid_mul(o, gate)
         return k.linear(o, w[f"{self.o_name}.weight"], w.get(f"{self.o_name}.bias"), deferred=True)
 
 

@@ -27,6 +27,32 @@ class ParamDecl:
     dtype: str = "model"
     sources: Optional[Tuple[Source, ...]] = None     # None: one tensor of the parameter's own name
     init: str = "normal"                             # random-weights mode: "normal" | "norm"
+    # A size of -1 in `shape` is one that the checkpoint's tensor decides (a rank that no configuration
+    # names); default_shape then says what random-weights mode draws.  Only for parameters of one source.
+    default_shape: Optional[Tuple[int, ...]] = None
+
+    def fits(self, shape) -> bool:
+        return len(shape) == len(self.shape) and all(w == -1 or w == g for w, g in zip(self.shape, shape))
+
+    @property
+    def drawn_shape(self) -> Tuple[int, ...]:
+        """The shape random-weights mode gives the parameter."""
+        if -1 not in self.shape:
+            return tuple(self.shape)
+        if self.default_shape is None or not self.fits(self.default_shape):
+            raise ValueError(f"a parameter of shape {self.shape} needs a default shape for its free sizes")
+        return tuple(self.default_shape)
+
+
+@dataclass
+class NormedAddend:
+    """A sublayer's output on its way into a float32 residual stream through a norm of its own:
+    the stream takes mult * x / sqrt(mean(x^2) + eps) * weight.  The norm that follows (the next
+    sublayer's, or the model's last) adds it while it reads the stream, in the same pass."""
+    x: object                         # [rows, width] of the element type (or a product left as partial sums)
+    weight: torch.Tensor              # [width]
+    eps: float
+    mult: float = 1.0
 
 
 @dataclass

@@ -18,6 +18,15 @@ norm as well: the block returns the two sublayer outputs as a list of addends wi
 it was before them, and the next block's norm (or the model's final norm) adds them.  The first
 block gets the embedding as its one addend.  A layer may have no feed-forward.
 
+"sandwich_residual": a norm before and a norm after every sublayer, the normed output times a
+constant added to the stream:
+    r <- r + c * post1(mixer(pre1(r)));   r <- r + c * post2(feed_forward(pre2(r)))
+The residual stream r is float32 whatever the element type.  The sum is deferred here too: a
+sublayer's output leaves the block as a NormedAddend (the output, the post-norm's weight and eps,
+the constant c), and the norm that follows norms it, adds it to the stream and norms the stream in
+one pass.  The first block gets the float32 stream itself from the embedding (an embedding with a
+scale gives one).  A layer may have no feed-forward.
+
 Interface of a block: forward(h, residual | None, batch, cache) -> (h, residual); h is a tensor,
 or a list of addends for a float32 stream.
 """
@@ -25,7 +34,9 @@ from __future__ import annotations
 
 from typing import Dict, Mapping
 
-from .base import BuildContext, Part
+import torch
+
+from .base import BuildContext, NormedAddend, Part
 from .registry import make_part, register_part
 
 
@@ -115,5 +126,60 @@ class ParallelResidualBlock(Part):
         return (a, self.feed_forward.forward(x, batch)), residual
 
 
+class SandwichResidualBlock(Part):
+    """params: residual_mult (default 1), parts and names by role: mixer_norm, mixer, mixer_post_norm, and,
+    where the layer has a feed-forward, feed_forward_norm, feed_forward, feed_forward_post_norm."""
+    ROLES = ("mixer_norm", "mixer", "mixer_post_norm", "feed_forward_norm", "feed_forward", "feed_forward_post_norm")
+
+    def __init__(self, params: Mapping, build: BuildContext):
+        super().__init__(params, build)
+        parts = params["parts"]
+        names = params["names"]
+        self.mult = float(params.get("residual_mult", 1.0))
+        self.dtype = build.dtype
+        has_ff = bool(parts.get("feed_forward"))
+        missing = [r for r in self.ROLES if r not in parts and (has_ff or not r.startswith("feed_forward"))]
+        if missing:
+            raise ValueError(f"sandwich_residual block: missing parts {missing}")
+        self.mixer_norm = make_part("norm", parts["mixer_norm"], build)
+        self.mixer = make_part("mixer", parts["mixer"], build)
+        self.mixer_post_norm = make_part("norm", parts["mixer_post_norm"], build)
+        self.feed_forward_norm = self.feed_forward = self.feed_forward_post_norm = None
+        if has_ff:
+            self.feed_forward_norm = make_part("norm", parts["feed_forward_norm"], build)
+            self.feed_forward = make_part("feed_forward", parts["feed_forward"], build)
+            self.feed_forward_post_norm = make_part("norm", parts["feed_forward_post_norm"], build)
+        self._children = {names[r]: getattr(self, r) for r in self.ROLES if getattr(self, r) is not None}
+
+    def children(self) -> Dict[str, Part]:
+        return self._children
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    @property
+    def replays_state_steps(self):
+        return self.mixer.replays_state_steps
+
+    def _through(self, post_norm, x) -> NormedAddend:
+        return NormedAddend(x, post_norm.weights["weight"], post_norm.eps, self.mult)
+
+    def forward(self, h, residual, batch, cache):
+        if residual is None:
+            # the first layer: h is the stream itself, float32, as the embedding made it
+            if not torch.is_tensor(h) or h.dtype != torch.float32:
+                raise ValueError("sandwich_residual block: the first layer takes the float32 stream from the embedding")
+            out = torch.empty(h.shape, dtype=self.dtype, device=h.device)
+            x, residual = self.mixer_norm.forward_add((), h, out=out)
+        else:
+            x, residual = self.mixer_norm.forward_add(tuple(h), residual)
+        a = self._through(self.mixer_post_norm, self.mixer.forward(x, batch, cache))
+        if self.feed_forward is None:
+            return (a,), residual
+        y, residual = self.feed_forward_norm.forward_add((a,), residual)
+        return (self._through(self.feed_forward_post_norm, self.feed_forward.forward(y, batch)),), residual
+
+
+register_part("block", "sandwich_residual", SandwichResidualBlock)
 register_part("block", "pre_norm_residual", PreNormResidualBlock)
 register_part("block", "parallel_residual", ParallelResidualBlock)

@@ -15,16 +15,22 @@ from .registry import register_part
 
 
 class TokenEmbedding(Part):
-    """weight [vocab, hidden]; rows are gathered by token id (embed_head.py:24,38)."""
+    """weight [vocab, hidden]; rows are gathered by token id (embed_head.py:24,38).  With the
+    parameter `scale` the rows are multiplied by that constant in float and leave as float32: the
+    start of a residual stream that is kept in float32."""
 
     def __init__(self, params: Mapping, build: BuildContext):
         super().__init__(params, build)
         self.vocab, self.hidden = int(params["vocab_size"]), int(params["hidden_size"])
+        scale = params.get("scale")
+        self.scale = None if scale is None else float(scale)
 
     def param_decls(self):
         return {"weight": ParamDecl((self.vocab, self.hidden))}
 
     def forward(self, ids):
+        if self.scale is not None:
+            return self.kernels.embedding_scaled(self.weights["weight"], ids, self.scale)
         return self.kernels.embedding(self.weights["weight"], ids)
 
 

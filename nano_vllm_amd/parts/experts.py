@@ -8,7 +8,11 @@
     scores (of its one score where groups hold one expert); only experts of the group_keep best groups
     can be chosen; of those the `top` with the largest scores are
     m = sum over the chosen e of (scale * s_e) expert_e(y)  +  shared(y)
-The weights are the scores themselves, not renormalised.  Routing is decided on the device and the
+The weights are the scores themselves, not renormalised.
+With routing "softmax_top" the router's logits (plus a bias, with router_bias) are compared as they are: the
+`top` largest are chosen and weighted by the softmax over the chosen logits alone (no groups, no scale).
+With gated = True an expert is the gated layer  Wd (act(Wg y) * (Wu y)).
+Routing is decided on the device and the
 experts' products run over the tokens sorted by expert, so a step never asks the host how many
 tokens an expert got: the same launches whatever the routing.
 """
@@ -46,8 +50,9 @@ class PlainMLP(Part):
 
 class MixtureOfExperts(Part):
     """params: hidden_size, num_experts, top, intermediate_size, scale, group_count, group_keep,
-    activation, shared (a PartSpec of a feed-forward, or None), and names: router_name, shared_name,
-    expert_name (a format with {} for the expert's number), up_name, down_name."""
+    activation, shared (a PartSpec of a feed-forward, or None), routing ("sigmoid_groups" | "softmax_top"),
+    router_bias (bool), gated (bool), and names: router_name, shared_name, expert_name (a format with {} for
+    the expert's number), gate_name, up_name, down_name."""
 
     kernel_modules = ("moe",)
 
@@ -64,6 +69,12 @@ class MixtureOfExperts(Part):
         self.activation = p.get("activation", "relu2")
         if self.activation not in ACTIVATIONS:
             raise ValueError(f"moe: unknown activation {self.activation!r}")
+        self.routing = p.get("routing", "sigmoid_groups")
+        if self.routing not in ("sigmoid_groups", "softmax_top"):
+            raise ValueError(f"moe: unknown routing {self.routing!r}")
+        self.router_bias = bool(p.get("router_bias", False))
+        self.gated = bool(p.get("gated", False))
+        self.gate_name = p.get("gate_name", "gate_proj")
         if self.experts % self.group_count or not 1 <= self.group_keep <= self.group_count:
             raise ValueError(f"moe: {self.experts} experts in {self.group_count} groups of which {self.group_keep} are kept")
         if not 1 <= self.top <= self.group_keep * (self.experts // self.group_count):
@@ -81,20 +92,35 @@ class MixtureOfExperts(Part):
     def param_decls(self) -> Dict[str, ParamDecl]:
         e, i, h = self.experts, self.inner, self.hidden
         name = self.expert_name.format
-        return {
+        if self.gated:
+            # an expert's gate rows, then its up rows: the first product makes both and gates in its epilogue
+            up = tuple(s for n in range(e) for s in (Source(f"{name(n)}.{self.gate_name}.weight", 2 * n * i, i),
+                                                     Source(f"{name(n)}.{self.up_name}.weight", (2 * n + 1) * i, i)))
+        else:
+            up = tuple(Source(f"{name(n)}.{self.up_name}.weight", n * i, i) for n in range(e))
+        decls = {
             f"{self.router_name}.weight": ParamDecl((e, h)),
             # the experts' matrices one below the other: expert n's rows are [n * rows, (n + 1) * rows)
-            "up.weight": ParamDecl((e * i, h), sources=tuple(
-                Source(f"{name(n)}.{self.up_name}.weight", n * i, i) for n in range(e))),
+            "up.weight": ParamDecl(((2 if self.gated else 1) * e * i, h), sources=up),
             "down.weight": ParamDecl((e * h, i), sources=tuple(
                 Source(f"{name(n)}.{self.down_name}.weight", n * h, h) for n in range(e))),
         }
+        if self.router_bias:
+            decls[f"{self.router_name}.bias"] = ParamDecl((e,), dtype="float32")
+        return decls
 
     def forward(self, x, batch=None):
         k, w = self.kernels, self.weights
         logits = k.linear(x, w[f"{self.router_name}.weight"], out_float32=True)
-        ids, weights = k.moe_route(logits, self.top, self.group_count, self.group_keep, self.scale)
+        if self.routing == "softmax_top":
+            ids, weights = k.moe_route(logits, self.top, 1, 1, 1.0, routing="softmax_top",
+                                       bias=w.get(f"{self.router_name}.bias"))
+        else:
+            ids, weights = k.moe_route(logits, self.top, self.group_count, self.group_keep, self.scale)
         shared = self.shared.forward(x, batch) if self.shared is not None else None
+        if self.gated:
+            return k.moe_experts(x, ids, weights, w["up.weight"], w["down.weight"], self.experts, self.activation,
+                                 add=shared, gated=True)
         return k.moe_experts(x, ids, weights, w["up.weight"], w["down.weight"], self.experts, self.activation, add=shared)
 
 

@@ -72,7 +72,7 @@ class Model:
     # ------------------------------------------------------------------ weights
     def set_param(self, name: str, tensor: torch.Tensor) -> None:
         owner, local, decl = self.param_table[name]
-        if tuple(tensor.shape) != tuple(decl.shape):
+        if not decl.fits(tuple(tensor.shape)):
             raise ValueError(f"parameter {name}: shape {tuple(tensor.shape)} is not {tuple(decl.shape)}")
         self.params[name] = tensor
         owner.weights[local] = tensor
@@ -108,7 +108,8 @@ class Model:
         return tuple(found)
 
     def num_parameters(self) -> int:
-        return sum(int(torch.tensor(d.shape).prod()) for _, _, d in self.param_table.values())
+        return sum(self.params[n].numel() if n in self.params else int(torch.tensor(d.drawn_shape).prod())
+                   for n, (_, _, d) in self.param_table.items())
 
     # ------------------------------------------------------------------ cache
     def cache_needs(self):

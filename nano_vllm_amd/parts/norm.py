@@ -6,7 +6,8 @@ residual sum (nanovllm/layers/layernorm.py:16-40).  Sizes and eps are parameters
 With weight_offset c the factor is (c + weight): c = 1 is the weight stored around zero.  A norm
 with an offset, and every norm that is handed a list of addends instead of one tensor, works on a
 residual stream kept in float32: the stream takes the sum of the addends, the norm is computed in
-float and rounded once to the element type.
+float and rounded once to the element type.  An addend may be a NormedAddend (parts.base): a sublayer's
+output that enters the stream through a norm of its own and a constant factor; the same pass does both norms.
 
 "dynamic_tanh": y = tanh(alpha * x) * weight + bias with one learned number alpha per norm: no mean,
 no variance, every entry by itself.  It works on a float32 residual stream (a list of addends, as

@@ -96,12 +96,14 @@ class PagedKV:
     are given back.  chunk: a query at position p reads positions >= floor(p / chunk) * chunk only
     (the sequence is cut into chunks counted from its position 0, and no query looks out of its
     own); pages wholly before the chunk of the next query are given back.  v_head_dim: the size of
-    a head's values where it is not head_dim."""
+    a head's values where it is not head_dim.  keep_first (with a window): every query also reads
+    the first keep_first positions of its sequence, whose pages are never given back."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     v_head_dim: Optional[int] = None
     chunk: Optional[int] = None
+    keep_first: int = 0
 
     @property
     def value_dim(self) -> int:

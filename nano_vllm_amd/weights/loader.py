@@ -59,6 +59,8 @@ def checkpoint_layout(model) -> Dict[str, Slot]:
             if called(full) in layout:
                 raise ValueError(f"two parameters claim the checkpoint tensor {called(full)!r}")
             layout[called(full)] = Slot(full, 0, decl.shape[0] if decl.shape else 1, tuple(decl.shape), True)
+        elif -1 in decl.shape:
+            raise ValueError(f"parameter {full!r}: a size left to the checkpoint goes with a single source")
         else:
             for src in decl.sources:
                 name = called(prefix + src.name)
@@ -104,8 +106,8 @@ def load_weights(model, folder: str) -> None:
                     continue
                 seen.add(name)
                 shape = tuple(f.get_slice(name).get_shape())
-                if shape != slot.shape:
-                    wrong.append((name, shape, slot.shape))
+                if len(shape) != len(slot.shape) or any(w != -1 and w != g for w, g in zip(slot.shape, shape)):
+                    wrong.append((name, shape, slot.shape))          # (-1: a size the tensor itself decides)
                     continue
                 t = f.get_tensor(name)
                 _, _, decl = model.param_table[slot.param]
@@ -113,8 +115,8 @@ def load_weights(model, folder: str) -> None:
                     if t.dtype in (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8) and decl.dtype != "int32":
                         wrong.append((name + f" (integer {t.dtype})", shape, slot.shape))
                         continue
-                    tensors[slot.param] = torch.empty(decl.shape, dtype=_param_dtype(decl, t.dtype, model.dtype),
-                                                      device=model.device)
+                    tensors[slot.param] = torch.empty(shape if slot.whole else decl.shape,
+                                                      dtype=_param_dtype(decl, t.dtype, model.dtype), device=model.device)
                 dst = tensors[slot.param]
                 dst = dst if slot.whole else dst.narrow(0, slot.row, slot.rows)
                 dst.copy_(t.to(dst.dtype))

@@ -40,6 +40,8 @@ def random_checkpoint(config_json: dict, seed: int, std: float = 0.02, norm_std:
     for name in sorted(layout):
         slot = layout[name]
         _, _, decl = model.param_table[slot.param]
+        if -1 in slot.shape:
+            slot = type(slot)(slot.param, slot.row, slot.rows, decl.drawn_shape, slot.whole)
         if decl.dtype == "int32":
             t = torch.randint(0, 2 ** 15, slot.shape, generator=gen, dtype=torch.int32)
         elif decl.init == "norm":
@@ -77,14 +79,14 @@ def fill_random_(model: Model, seed: int, std: float = 0.02, norm_std: float = 0
         gen.manual_seed((seed * 1000003 + zlib.crc32(name.encode())) % (2 ** 63))
         dtype = torch.int32 if decl.dtype == "int32" else (torch.float32 if decl.dtype == "float32" else model.dtype)
         if decl.dtype == "int32":
-            t = torch.randint(0, 2 ** 15, decl.shape, generator=gen, dtype=torch.int32, device=model.device)
+            t = torch.randint(0, 2 ** 15, decl.drawn_shape, generator=gen, dtype=torch.int32, device=model.device)
         elif decl.init == "norm":
-            t = torch.ones(decl.shape, dtype=torch.float32, device=model.device)
+            t = torch.ones(decl.drawn_shape, dtype=torch.float32, device=model.device)
             if norm_std > 0:
-                t += norm_std * torch.randn(decl.shape, generator=gen, dtype=torch.float32, device=model.device)
+                t += norm_std * torch.randn(decl.drawn_shape, generator=gen, dtype=torch.float32, device=model.device)
             t = t.to(dtype)
         else:
-            t = torch.empty(decl.shape, dtype=dtype, device=model.device)
+            t = torch.empty(decl.drawn_shape, dtype=dtype, device=model.device)
             t.normal_(0.0, std, generator=gen)
         model.set_param(name, t)
     model.finish_weights()

@@ -51,6 +51,9 @@ class TorchKernels:
 
     gather_rows = embedding
 
+    def embedding_scaled(self, table, ids, scale):
+        return table[ids.long()].float() * scale
+
     # norms (layernorm.py:16-40)
     def rms_norm(self, x, weight, eps, out=None):
         xf = x.float()
@@ -74,13 +77,20 @@ class TorchKernels:
     def stream_rms_norm(self, addends, residual, weight, eps, offset=0.0, out=None):
         """The float32 residual stream takes the sum of the addends; its norm, in float, rounded once."""
         add = None
+        dt = out.dtype if out is not None else None
         for a in addends:
-            add = a.float() if add is None else add + a.float()
+            if hasattr(a, "mult"):          # an addend that enters through a norm of its own, times a constant
+                x = a.x.float()
+                dt = dt or a.x.dtype
+                x = a.mult * (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + a.eps) * a.weight.float())
+            else:
+                x = a.float()
+                dt = dt or a.dtype
+            add = x if add is None else add + x
         if residual is None:
             residual = add.clone()
         elif add is not None:
             residual += add
-        dt = addends[0].dtype if addends else out.dtype
         y = (residual * torch.rsqrt(residual.pow(2).mean(-1, keepdim=True) + eps) * (offset + weight.float())).to(dt)
         if out is not None:
             out.copy_(y)
@@ -137,9 +147,14 @@ class TorchKernels:
         return y
 
     # routed feed-forward
-    def moe_route(self, logits, top, group_count, group_keep, scale):
-        """int32 [T, top] experts and float32 [T, top] weights (scale * sigmoid score) of every token."""
+    def moe_route(self, logits, top, group_count, group_keep, scale, routing="sigmoid_groups", bias=None):
+        """int32 [T, top] experts and float32 [T, top] weights (scale * sigmoid score) of every token; with
+        routing "softmax_top" the largest logits (plus bias) and the softmax over them alone."""
         T, E = logits.shape
+        if routing == "softmax_top":
+            z = logits.float() + (bias.float() if bias is not None else 0.0)
+            best = z.topk(top, dim=-1)
+            return best.indices.to(torch.int32), torch.softmax(best.values, dim=-1)
         s = torch.sigmoid(logits.float())
         per = E // group_count
         grouped = s.view(T, group_count, per)
@@ -151,15 +166,22 @@ class TorchKernels:
         ids = masked.topk(top, dim=-1).indices
         return ids.to(torch.int32), (s.gather(1, ids) * scale).float()
 
-    def moe_experts(self, x, ids, weights, up, down, num_experts, act="relu2", add=None):
-        """sum over a token's experts e of weight * act(x Wu_e^T) Wd_e^T (+ add); up [E * ff, K], down [E * K, ff]."""
+    def moe_experts(self, x, ids, weights, up, down, num_experts, act="relu2", add=None, gated=False):
+        """sum over a token's experts e of weight * act(x Wu_e^T) Wd_e^T (+ add); up [E * ff, K], down [E * K, ff].
+        gated: up [E * 2 ff, K] holds an expert's gate rows, then its up rows, and the hidden layer is
+        act(x Wg_e^T) * (x Wu_e^T)."""
         T, K = x.shape
-        ff = up.shape[0] // num_experts
+        ff = up.shape[0] // num_experts // (2 if gated else 1)
         out = torch.zeros((T, K), dtype=torch.float32, device=x.device)
         for e in range(num_experts):
             hit = ids == e
             rows = hit.any(-1)
-            if bool(rows.any()):
+            if bool(rows.any()) and gated:
+                both = x[rows].float() @ up[2 * e * ff:2 * (e + 1) * ff].float().T
+                h = (self._activation(both[:, :ff], act) * both[:, ff:]).to(x.dtype).float()
+                y = (h @ down[e * K:(e + 1) * K].float().T).to(x.dtype).float()
+                out[rows] += (weights * hit)[rows].sum(-1, keepdim=True) * y
+            elif bool(rows.any()):
                 h = self._activation((x[rows].float() @ up[e * ff:(e + 1) * ff].float().T), act).to(x.dtype).float()
                 y = (h @ down[e * K:(e + 1) * K].float().T).to(x.dtype).float()
                 out[rows] += (weights * hit)[rows].sum(-1, keepdim=True) * y
@@ -253,7 +275,7 @@ class TorchKernels:
         return torch.cat((ang.cos(), ang.sin()), dim=-1)
 
     def qk_rownorm_store(self, qkv, num_heads, num_kv_heads, head_dim, v_head_dim, q_weight, k_weight, eps,
-                         positions, temp_coef, temp_every, slots, k_cache, v_cache, rot_table=None):
+                         positions, temp_coef, temp_every, slots, k_cache, v_cache, rot_table=None, norm_per_head=False):
         """q and k normed over the whole projection, q times its position's temperature, both rotated by
         the rows of rot_table (one per token: cosines, then sines, for the first channels of a head),
         k and v stored."""
@@ -269,9 +291,14 @@ class TorchKernels:
             cos, sin = rot_table[:, None, : R // 2], rot_table[:, None, R // 2:]
             a, b = x[..., : R // 2], x[..., R // 2:R]
             return torch.cat((a * cos - b * sin, b * cos + a * sin, x[..., R:]), dim=-1).reshape(T, heads * head_dim)
+        def normed(x, heads, w):
+            if norm_per_head:               # every head by itself, with a weight of the head's size
+                x = x.reshape(T, heads, head_dim)
+                return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()).reshape(T, heads * head_dim)
+            return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()
         q = qkv[:, :qd].float()
         if q_weight is not None:
-            q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_weight.float()
+            q = normed(q, num_heads, q_weight)
         if temp_coef:
             steps = torch.div(positions.long() + 1, int(temp_every), rounding_mode="floor").float()
             q = q * (1.0 + temp_coef * torch.log(steps + 1.0))[:, None]
@@ -279,7 +306,7 @@ class TorchKernels:
         if num_kv_heads:
             k = qkv[:, qd:qd + kd].float()
             if k_weight is not None:
-                k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_weight.float()
+                k = normed(k, num_kv_heads, k_weight)
             qkv[:, qd:qd + kd] = turn(k, num_kv_heads).to(dt)
             if k_cache is not None:
                 page_size, vt = k_cache.shape[2], v_cache.shape[4]
@@ -289,6 +316,57 @@ class TorchKernels:
                 k_cache[page, :, off, :] = qkv[:, qd:qd + kd].reshape(T, num_kv_heads, head_dim)[ok]
                 v_cache[page, :, off // vt, :, off % vt] = qkv[:, qd + kd:].reshape(T, num_kv_heads, v_head_dim)[ok]
         return qkv[:, :qd]
+
+    def sigmoid_mul(self, x, gate, out=None):
+        """x * sigmoid(gate), entry by entry; in place unless out is given."""
+        y = (x.float() * torch.sigmoid(gate.float())).to(x.dtype)
+        out = x if out is None else out
+        out.copy_(y)
+        return out
+
+    def channel_delta(self, proj, decay_in, gate_in, heads, kv_heads, dim, vdim, taps, conv_w, dt_bias, a_log, norm_w,
+                      eps, conv_state, s_state, batch, out=None):
+        """Token by token: the three convolutions over the request's last inputs, unit-norm q and k, beta, the
+        decay per key channel, S <- diag(a) S, u = beta (v - S^T k), S <- S + k u^T, o = S^T q, then the norm per
+        head and the gate."""
+        T = proj.shape[0]
+        qk, vv = kv_heads * dim, heads * vdim
+        C = 2 * qk + vv
+        p = proj.float()
+        raw, beta = p[:, :C], torch.sigmoid(p[:, C:C + heads])
+        step = torch.nn.functional.softplus(decay_in.float() + dt_bias.float(), threshold=1e9).reshape(T, heads, dim)
+        decay = torch.exp(-torch.exp(a_log.float())[None, :, None] * step)
+        o = torch.zeros((T, heads, vdim), dtype=torch.float32, device=proj.device)
+        per = heads // kv_heads
+        slots = batch.state_slots.tolist()
+        t = 0
+        for s, (start, n) in enumerate(zip(batch.starts, batch.q_lens)):
+            slot = slots[s]
+            hist = conv_state[slot].clone() if start > 0 else torch.zeros_like(conv_state[slot])      # [C, taps - 1]
+            S = s_state[slot].clone() if start > 0 else torch.zeros_like(s_state[slot])               # [heads, dim, vdim]
+            for i in range(t, t + n):
+                window = torch.cat((hist, raw[i][:, None]), dim=1)                                    # [C, taps]
+                c = (window * conv_w.float()).sum(-1)
+                c = c * torch.sigmoid(c)
+                hist = window[:, 1:]
+                q = c[:qk].reshape(kv_heads, dim)
+                k = c[qk:2 * qk].reshape(kv_heads, dim)
+                v = c[2 * qk:].reshape(heads, vdim)
+                q = (q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6) * dim ** -0.5).repeat_interleave(per, 0)
+                k = (k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)).repeat_interleave(per, 0)
+                S = decay[i][:, :, None] * S
+                u = beta[i][:, None] * (v - torch.einsum("hdv,hd->hv", S, k))
+                S = S + k[:, :, None] * u[:, None, :]
+                o[i] = torch.einsum("hdv,hd->hv", S, q)
+            conv_state[slot] = hist
+            s_state[slot] = S
+            t += n
+        o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
+        y = (o.reshape(T, vv) * torch.sigmoid(gate_in.float())).to(proj.dtype)
+        if out is not None:
+            out.copy_(y)
+            return out
+        return y
 
     RETENTION_CHUNK = 4
 
@@ -371,7 +449,7 @@ class TorchKernels:
 
     # attention (attention.py:64-75): token by token through the block table
     def paged_attention(self, q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, batch, group, scale,
-                        window=None, out=None, v_head_dim=None, sinks=None, chunk=None):
+                        window=None, out=None, v_head_dim=None, sinks=None, chunk=None, softcap=None, keep_first=0):
         T = q.shape[0]
         D, G = head_dim, num_heads // num_kv_heads
         DV = v_head_dim or head_dim
@@ -385,6 +463,8 @@ class TorchKernels:
             if chunk:
                 first = max(first, pos // chunk * chunk)
             js = torch.arange(first, pos + 1, device=q.device)
+            if window and keep_first and first > 0:       # the sequence's first positions stay in sight
+                js = torch.cat((torch.arange(0, min(keep_first, first), device=q.device), js))
             pages = tables[seq].long()[js // page_size]
             assert bool((pages >= 0).all()), "a visible key has no page"
             offs = js % page_size
@@ -394,6 +474,8 @@ class TorchKernels:
             qt = q[t].float().reshape(num_heads, D)
             for h in range(num_heads):
                 s = (keys[:, h // G] @ qt[h]) * scale
+                if softcap:
+                    s = softcap * torch.tanh(s / softcap)
                 if sinks is not None:       # one more term in the denominator: a key without a value
                     p = torch.softmax(torch.cat((s, sinks[h:h + 1].float())), dim=0)[:-1]
                 else:
