@@ -103,4 +103,28 @@ NVA_EXPORT int NVA_NAME(nva_act)(const void* x, int64_t x_stride, void* out, int
     return nva_check_launch("act");
 }
 
+// A gate on finished outputs: out[t, i] = x[t, i] * sigmoid(g[t, i]), in float, rounded once (out may be x).
+template <typename T>
+__global__ void __launch_bounds__(256)
+sigmoid_mul_kernel(const T* __restrict__ x, int64_t x_stride, const T* __restrict__ g, int64_t g_stride, T* __restrict__ out,
+                   int64_t out_stride, int64_t rows, int width) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= rows * width) return;
+    const int64_t r = idx / width;
+    const int i = (int)(idx % width);
+    const float gate = 1.f / (1.f + nva_exp(-to_float(g[r * g_stride + i])));
+    out[r * out_stride + i] = from_float<T>(to_float(x[r * x_stride + i]) * gate);
+}
+
+NVA_EXPORT int NVA_NAME(nva_sigmoid_mul)(const void* x, int64_t x_stride, const void* g, int64_t g_stride, void* out,
+                                         int64_t out_stride, int64_t rows, int width, hipStream_t stream) {
+    if (rows == 0) return 0;
+    if (rows < 0 || width <= 0 || !x || !g || !out) return nva_fail("sigmoid_mul: bad shape rows=%lld width=%d", (long long)rows, width);
+    const int64_t total = rows * width;
+    if ((total + 255) / 256 > 0x7fffffff) return nva_fail("sigmoid_mul: too many entries");
+    hipLaunchKernelGGL((sigmoid_mul_kernel<elem_t>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                       (const elem_t*)x, x_stride, (const elem_t*)g, g_stride, (elem_t*)out, out_stride, rows, width);
+    return nva_check_launch("sigmoid_mul");
+}
+
 NVA_DEFINE_LAST_ERROR(nva_activation)

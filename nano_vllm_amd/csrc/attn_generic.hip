@@ -15,6 +15,9 @@
 // The values may have a size of their own, DV (V [pages, Hkv, page / vt, DV, vt], output rows of Hq * DV).
 // sinks, float [Hq] or null: a head's softmax has one more term exp(sink_h) in its denominator, a key
 // without a value that every query sees once; the running maximum starts at sink_h with a sum of 1.
+// softcap > 0: s_j <- softcap * tanh(s_j / softcap) after the scale.  keep_first > 0 (with a window): the keys
+// at positions < keep_first stay visible to every query, however far back; the per-token kernel walks them
+// first, then the window.
 //
 // Portions of prompts have a second kernel with the same arithmetic, operation for operation (the
 // results are the same bits): a workgroup takes 32 query rows of one request and one head, and the
@@ -34,7 +37,8 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
                                const int32_t* __restrict__ block_tables, int table_stride,
                                const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
                                int num_q_heads, int num_kv_heads, int head_dim, int v_dim, int page_size, float scale,
-                               int window, int chunk, const float* __restrict__ sinks, int32_t* error_flag) {
+                               int window, int chunk, int keep_first, float softcap, const float* __restrict__ sinks,
+                               int32_t* error_flag) {
     __shared__ float q_s[ATT_MAX_D];
     __shared__ float p_s[NVA_WAVE];
     __shared__ int64_t v_off_s[NVA_WAVE];
@@ -59,11 +63,15 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
     const bool vec = head_dim % 8 == 0;
     const int vt = nva_v_tile(page_size);
 
-    for (int base = chunk > 0 ? first / NVA_WAVE * NVA_WAVE : first; base <= pos; base += NVA_WAVE) {
+    // the kept first positions that the window has passed, [0, kept_end), then the window (or chunk) up to pos
+    const int kept_end = window > 0 && keep_first > 0 ? min(keep_first, first) : 0;
+    for (int part = kept_end > 0 ? 0 : 1; part < 2; ++part) {
+    const int lo = part == 0 ? 0 : first, hi = part == 0 ? kept_end - 1 : pos;
+    for (int base = part == 1 && chunk > 0 ? first / NVA_WAVE * NVA_WAVE : lo; base <= hi; base += NVA_WAVE) {
         const int j = base + lane;
         float s = -INFINITY;
         int64_t v_off = 0;
-        if (j <= pos && j >= first) {
+        if (j <= hi && j >= lo) {
             const int page = table[j / page_size];
             const int off = j % page_size;
             if (page < 0) {
@@ -94,6 +102,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
                     for (int d = 0; d < head_dim; ++d) dot += q_s[d] * to_float(krow[d]);
                 }
                 s = dot * scale;
+                if (softcap > 0.f) s = softcap * tanhf(s / softcap);
             }
         }
         const float m_new = fmaxf(m_run, wave_max(s));
@@ -107,7 +116,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
         p_s[lane] = p;
         v_off_s[lane] = v_off;
         __syncthreads();
-        const int valid = pos - base + 1 < NVA_WAVE ? pos - base + 1 : NVA_WAVE;
+        const int valid = hi - base + 1 < NVA_WAVE ? hi - base + 1 : NVA_WAVE;
 #pragma unroll
         for (int i = 0; i < ATT_ACC; ++i) {
             const int d = lane + i * NVA_WAVE;
@@ -133,6 +142,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
                 acc[i] = a;
             }
         }
+    }
     }
     const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
     T* orow = out + t * out_stride + (int64_t)h * v_dim;
@@ -162,8 +172,8 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
                              const int32_t* __restrict__ block_tables, int table_stride,
                              const int32_t* __restrict__ cu_seqlens_q, const int32_t* __restrict__ kv_lens,
                              const int32_t* __restrict__ tiles, int num_q_heads, int num_kv_heads, int head_dim,
-                             int v_dim, int page_size, float scale, int chunk, const float* __restrict__ sinks,
-                             int32_t* error_flag) {
+                             int v_dim, int page_size, float scale, int chunk, float softcap,
+                             const float* __restrict__ sinks, int32_t* error_flag) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     __shared__ int64_t k_off_s[NVA_WAVE], v_off_s[NVA_WAVE];       // of a chunk's keys; -1: the key has no page
     constexpr int ROWS_PER_WAVE = ATT_ROWS / ATT_TILED_WAVES;
@@ -322,7 +332,9 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 const int rr = 4 * quad + t;
-                const float s = base + lane <= pos4[t] && base + lane >= first4[t] && key_ok ? dot[t] * scale : -INFINITY;
+                float s = dot[t] * scale;
+                if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+                if (!(base + lane <= pos4[t] && base + lane >= first4[t] && key_ok)) s = -INFINITY;
                 const float m_new = fmaxf(m_run[rr], wave_max(s));
                 p[t] = (s == -INFINITY) ? 0.f : nva_exp(s - m_new);
                 const float correction = (m_run[rr] == -INFINITY) ? 0.f : nva_exp(m_run[rr] - m_new);
@@ -383,7 +395,7 @@ NVA_EXPORT int NVA_NAME(nva_paged_attention_tiled)(
     const void* q, int64_t q_stride, void* out, int64_t out_stride, const void* k_cache, const void* v_cache,
     const int32_t* block_tables, int table_stride, const int32_t* cu_seqlens_q, const int32_t* kv_lens,
     const int32_t* tiles, int64_t num_tiles, int num_q_heads, int num_kv_heads, int head_dim, int v_dim,
-    int page_size, float scale, int chunk, const float* sinks, int32_t* error_flag, hipStream_t stream) {
+    int page_size, float scale, int chunk, float softcap, const float* sinks, int32_t* error_flag, hipStream_t stream) {
     if (num_tiles == 0) return 0;
     if (chunk < 0) return nva_fail("paged_attention_tiled: negative chunk");
     if (head_dim <= 0 || head_dim > ATT_TILED_MAX_D || v_dim <= 0 || v_dim > ATT_TILED_MAX_D) {
@@ -406,7 +418,7 @@ NVA_EXPORT int NVA_NAME(nva_paged_attention_tiled)(
     hipLaunchKernelGGL(kernel, grid, dim3(ATT_TILED_WAVES * NVA_WAVE), lds, stream, (const elem_t*)q, q_stride,
                        (elem_t*)out, out_stride, (const elem_t*)k_cache, (const elem_t*)v_cache, block_tables,
                        table_stride, cu_seqlens_q, kv_lens, tiles, num_q_heads, num_kv_heads, head_dim, v_dim,
-                       page_size, scale, chunk, sinks, error_flag);
+                       page_size, scale, chunk, softcap, sinks, error_flag);
     return nva_check_launch("paged_attention_tiled");
 }
 
@@ -414,7 +426,7 @@ NVA_EXPORT int NVA_NAME(nva_paged_attention_generic)(
     const void* q, int64_t q_stride, void* out, int64_t out_stride, const void* k_cache, const void* v_cache,
     const int32_t* block_tables, int table_stride, const int32_t* token_seq, const int32_t* positions,
     int64_t tokens, int num_q_heads, int num_kv_heads, int head_dim, int v_dim, int page_size, float scale,
-    int window, int chunk, const float* sinks, int32_t* error_flag, hipStream_t stream) {
+    int window, int chunk, int keep_first, float softcap, const float* sinks, int32_t* error_flag, hipStream_t stream) {
     if (tokens == 0) return 0;
     if (tokens < 0 || tokens > 0x7fffffff) return nva_fail("paged_attention: bad token count %lld", (long long)tokens);
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads || num_q_heads > 65535)
@@ -422,12 +434,12 @@ NVA_EXPORT int NVA_NAME(nva_paged_attention_generic)(
     if (head_dim <= 0 || head_dim > ATT_MAX_D || v_dim <= 0 || v_dim > ATT_MAX_D)
         return nva_fail("paged_attention: head sizes %d / %d are outside 1..%d", head_dim, v_dim, ATT_MAX_D);
     if (page_size <= 0 || table_stride <= 0) return nva_fail("paged_attention: bad page size or table width");
-    if (window < 0 || chunk < 0) return nva_fail("paged_attention: negative window or chunk");
+    if (window < 0 || chunk < 0 || keep_first < 0) return nva_fail("paged_attention: negative window, chunk or kept positions");
     dim3 grid((unsigned)tokens, (unsigned)num_q_heads);
     hipLaunchKernelGGL(paged_attention_generic_kernel<elem_t>, grid, dim3(NVA_WAVE), 0, stream, (const elem_t*)q,
                        q_stride, (elem_t*)out, out_stride, (const elem_t*)k_cache, (const elem_t*)v_cache,
                        block_tables, table_stride, token_seq, positions, num_q_heads, num_kv_heads, head_dim,
-                       v_dim, page_size, scale, window, chunk, sinks, error_flag);
+                       v_dim, page_size, scale, window, chunk, keep_first, softcap, sinks, error_flag);
     return nva_check_launch("paged_attention_generic");
 }
 

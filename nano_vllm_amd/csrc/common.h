@@ -138,7 +138,7 @@ __device__ __forceinline__ float nva_gate_act(int act, float g) {
     if (act == 1) return fmaxf(g, 0.f);
     if (act == 3) { const float r = fmaxf(g, 0.f); return r * r; }
     if (act == 2) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
-    return g / (1.f + __expf(-g));
+    return g / (1.f + nva_exp(-g));
 }
 
 // ---------------------------------------------------------------------------- split products

@@ -1,0 +1,262 @@
+// The gated delta rule with a decay per key channel, after its projections: a linear attention over a state
+// of fixed size per request that forgets channel by channel and, at every token, is corrected towards the value
+// its key should read out.
+//
+//   proj [T, 2 G D + H DV + H] = [q | k | v | b]        elements; G query/key heads of D, H value heads of DV
+//   q, k, v <- silu(sum over the last `taps` tokens of w[c][j] * input[c])      per channel c, no bias; the inputs
+//              before a portion come from the request's kept inputs (conv_state), zeros before its start
+//   q <- q / sqrt(sum(q^2) + 1e-6) * D^-1/2,  k <- k / sqrt(sum(k^2) + 1e-6)    per head
+//   beta = sigmoid(b)                                                            per value head
+//   a = exp(-exp(a_log[h]) * softplus(decay_in[h][d] + dt_bias[h][d]))          per value head and key channel
+//   per value head h, with its query/key head h / (H / G), S [D, DV]:
+//       S <- diag(a) S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
+//   y = o / sqrt(mean(o^2) + eps) * norm_w * sigmoid(gate_in)                   per head, norm_w [DV]
+//
+// Everything after the projections is float whatever the element type (the convolutions' sums, the unit norms,
+// softplus and the exponentials by the accurate routines, the state, the read-out, the norm and the gate); y is
+// rounded once.  A token's sums run in an order that neither the portion's cut nor the batch changes: the
+// recurrence goes token by token, a thread holding one column of S in registers.
+//
+//   delta_prepare     one workgroup a token: the convolutions, unit norms, beta and the decay, written as floats
+//   delta_keep        the request's new kept inputs (its last taps - 1), after delta_prepare has read the old ones
+//   delta_scan        one wave per (request, head, 64 columns of S): the recurrence over the portion's tokens, the
+//                     tokens' q, k and a staged in LDS a batch at a time, v and beta asked for a batch ahead
+//   delta_finish      one wave per (token, head): the norm and the gate
+#include "common.h"
+
+#define DELTA_MAX_TAPS 16
+#define DELTA_BATCH 8            // tokens whose q, k and a lie in LDS at a time
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+delta_prepare_kernel(const T* __restrict__ proj, int64_t stride, const float* __restrict__ decay_in,
+                     const T* __restrict__ conv_w, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+                     const float* __restrict__ conv_state, const int32_t* __restrict__ token_seq,
+                     const int32_t* __restrict__ cu_seqlens_q, const int32_t* __restrict__ seq_starts,
+                     const int32_t* __restrict__ state_slots, int heads, int kv_heads, int dim, int vdim, int taps,
+                     float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ vf, float* __restrict__ decay,
+                     float* __restrict__ beta) {
+    extern __shared__ __attribute__((aligned(16))) float row_s[];      // the token's q and k after convolution and silu
+    const int64_t t = blockIdx.x;
+    const int seq = token_seq[t];
+    const int begin = cu_seqlens_q[seq];
+    const int local = (int)t - begin;                                   // the token's place in its portion
+    const bool has_past = seq_starts[seq] > 0;
+    const int slot = state_slots[seq];
+    const int qk = kv_heads * dim, vv = heads * vdim, channels = 2 * qk + vv;
+    const int tid = threadIdx.x;
+    for (int c = tid; c < channels; c += blockDim.x) {
+        float sum = 0.f;
+        for (int j = 0; j < taps; ++j) {
+            const int src = local - (taps - 1) + j;                     // < 0: before the portion
+            float x = 0.f;
+            if (src >= 0) x = to_float(proj[(int64_t)(begin + src) * stride + c]);
+            else if (has_past) x = conv_state[((int64_t)slot * channels + c) * (taps - 1) + (taps - 1 + src)];
+            sum += to_float(conv_w[(int64_t)c * taps + j]) * x;
+        }
+        const float y = sum / (1.f + expf(-sum));
+        if (c < 2 * qk) row_s[c] = y; else vf[t * vv + (c - 2 * qk)] = y;
+    }
+    __syncthreads();
+    // unit norms per head: q heads first, then k heads
+    const int wave = tid / NVA_WAVE, lane = tid % NVA_WAVE, nwaves = blockDim.x / NVA_WAVE;
+    for (int hh = wave; hh < 2 * kv_heads; hh += nwaves) {
+        const float* x = row_s + hh * dim;
+        float ss = 0.f;
+        for (int d = lane; d < dim; d += NVA_WAVE) ss += x[d] * x[d];
+        ss = wave_sum(ss);
+        float scale = 1.f / sqrtf(ss + 1e-6f);
+        const bool is_q = hh < kv_heads;
+        if (is_q) scale *= 1.f / sqrtf((float)dim);
+        float* dst = is_q ? qn + t * qk + hh * dim : kn + t * qk + (hh - kv_heads) * dim;
+        for (int d = lane; d < dim; d += NVA_WAVE) dst[d] = x[d] * scale;
+    }
+    for (int i = tid; i < heads * dim; i += blockDim.x) {
+        const float z = decay_in[t * (int64_t)(heads * dim) + i] + dt_bias[i];
+        const float step = z > 20.f ? z : log1pf(expf(z));
+        decay[t * (int64_t)(heads * dim) + i] = expf(-expf(a_log[i / dim]) * step);
+    }
+    for (int h = tid; h < heads; h += blockDim.x)
+        beta[t * heads + h] = 1.f / (1.f + expf(-to_float(proj[t * stride + channels + h])));
+}
+
+// One thread a (request, channel): the request's last taps - 1 inputs, from the portion where it is long enough,
+// else from what was kept before (zeros at a request's start).
+template <typename T>
+__global__ void __launch_bounds__(256)
+delta_keep_kernel(const T* __restrict__ proj, int64_t stride, float* __restrict__ conv_state,
+                  const int32_t* __restrict__ cu_seqlens_q, const int32_t* __restrict__ seq_starts,
+                  const int32_t* __restrict__ state_slots, int channels, int taps) {
+    const int seq = blockIdx.y;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= channels) return;
+    const int begin = cu_seqlens_q[seq], n = cu_seqlens_q[seq + 1] - begin;
+    const bool has_past = seq_starts[seq] > 0;
+    float* kept = conv_state + ((int64_t)state_slots[seq] * channels + c) * (taps - 1);
+    float fresh[DELTA_MAX_TAPS];
+    for (int i = 0; i < taps - 1; ++i) {
+        const int src = n - (taps - 1) + i;
+        fresh[i] = src >= 0 ? to_float(proj[(int64_t)(begin + src) * stride + c]) : has_past ? kept[taps - 1 + src] : 0.f;
+    }
+    for (int i = 0; i < taps - 1; ++i) kept[i] = fresh[i];
+}
+
+// One wave per (request, head, 64 columns of S).  A thread holds its column's DMAX rows (rows beyond D: zeros, with
+// q, k and a staged as zeros).  Per token, in this order: S <- a S, u = beta (v - S^T k), S <- S + k u, o = S^T q; the
+// two sums over the rows run as four chains each, in an order that depends on D alone.
+template <int DMAX>
+__global__ void __launch_bounds__(NVA_WAVE)
+delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vf,
+                  const float* __restrict__ decay, const float* __restrict__ beta, float* __restrict__ o_raw,
+                  float* __restrict__ state, const int32_t* __restrict__ cu_seqlens_q,
+                  const int32_t* __restrict__ seq_starts, const int32_t* __restrict__ state_slots, int heads,
+                  int kv_heads, int dim, int vdim) {
+    __shared__ __attribute__((aligned(16))) float q_s[DELTA_BATCH][DMAX], k_s[DELTA_BATCH][DMAX], a_s[DELTA_BATCH][DMAX];
+    __shared__ float beta_s[DELTA_BATCH];
+    const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int col = blockIdx.z * NVA_WAVE + lane;
+    const bool live = col < vdim;
+    const int g = h / (heads / kv_heads);
+    const int begin = cu_seqlens_q[seq], n = cu_seqlens_q[seq + 1] - begin;
+    const int qk = kv_heads * dim, vv = heads * vdim, hd = heads * dim;
+    float* S_g = state + (((int64_t)state_slots[seq] * heads + h) * dim) * vdim + col;
+    float S[DMAX];
+    const bool has_past = seq_starts[seq] > 0;
+#pragma unroll
+    for (int i = 0; i < DMAX; ++i) S[i] = has_past && live && i < dim ? S_g[(int64_t)i * vdim] : 0.f;
+
+    float v_next[DELTA_BATCH];
+#pragma unroll
+    for (int b = 0; b < DELTA_BATCH; ++b) v_next[b] = live && b < n ? vf[(int64_t)(begin + b) * vv + h * vdim + col] : 0.f;
+    for (int t0 = 0; t0 < n; t0 += DELTA_BATCH) {
+        const int nb = min(DELTA_BATCH, n - t0);
+        __syncthreads();                                               // the batch before is done with
+        for (int i = lane; i < DELTA_BATCH * DMAX; i += NVA_WAVE) {
+            const int b = i / DMAX, d = i % DMAX;
+            const bool ok = b < nb && d < dim;
+            const int64_t tok = begin + t0 + b;
+            q_s[b][d] = ok ? qn[tok * qk + g * dim + d] : 0.f;
+            k_s[b][d] = ok ? kn[tok * qk + g * dim + d] : 0.f;
+            a_s[b][d] = ok ? decay[tok * hd + h * dim + d] : 0.f;
+        }
+        if (lane < DELTA_BATCH) beta_s[lane] = lane < nb ? beta[(int64_t)(begin + t0 + lane) * heads + h] : 0.f;
+        float v_now[DELTA_BATCH];
+#pragma unroll
+        for (int b = 0; b < DELTA_BATCH; ++b) {
+            v_now[b] = v_next[b];
+            const int tn = t0 + DELTA_BATCH + b;                        // the batch after: asked for now
+            v_next[b] = live && tn < n ? vf[(int64_t)(begin + tn) * vv + h * vdim + col] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int b = 0; b < DELTA_BATCH; ++b) {
+            if (b >= nb) break;
+            float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+#pragma unroll
+            for (int i = 0; i < DMAX; i += 4) {
+                const float4 a = *reinterpret_cast<const float4*>(&a_s[b][i]);
+                const float4 k = *reinterpret_cast<const float4*>(&k_s[b][i]);
+                S[i] *= a.x; S[i + 1] *= a.y; S[i + 2] *= a.z; S[i + 3] *= a.w;
+                d0 += S[i] * k.x; d1 += S[i + 1] * k.y; d2 += S[i + 2] * k.z; d3 += S[i + 3] * k.w;
+            }
+            const float u = beta_s[b] * (v_now[b] - ((d0 + d1) + (d2 + d3)));
+            float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+#pragma unroll
+            for (int i = 0; i < DMAX; i += 4) {
+                const float4 k = *reinterpret_cast<const float4*>(&k_s[b][i]);
+                const float4 q = *reinterpret_cast<const float4*>(&q_s[b][i]);
+                S[i] += k.x * u; S[i + 1] += k.y * u; S[i + 2] += k.z * u; S[i + 3] += k.w * u;
+                o0 += S[i] * q.x; o1 += S[i + 1] * q.y; o2 += S[i + 2] * q.z; o3 += S[i + 3] * q.w;
+            }
+            if (live) o_raw[(int64_t)(begin + t0 + b) * vv + h * vdim + col] = (o0 + o1) + (o2 + o3);
+        }
+    }
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < DMAX; ++i)
+            if (i < dim) S_g[(int64_t)i * vdim] = S[i];
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(NVA_WAVE)
+delta_finish_kernel(const float* __restrict__ o_raw, const T* __restrict__ gate, int64_t gate_stride,
+                    const float* __restrict__ norm_w, float eps, T* __restrict__ out, int64_t out_stride, int heads,
+                    int vdim) {
+    const int64_t t = blockIdx.x;
+    const int h = blockIdx.y, lane = threadIdx.x;
+    const float* o = o_raw + (t * heads + h) * (int64_t)vdim;
+    float ss = 0.f;
+    for (int d = lane; d < vdim; d += NVA_WAVE) ss += o[d] * o[d];
+    ss = wave_sum(ss);
+    const float scale = 1.f / sqrtf(ss / (float)vdim + eps);
+    for (int d = lane; d < vdim; d += NVA_WAVE) {
+        const float gt = 1.f / (1.f + expf(-to_float(gate[t * gate_stride + h * vdim + d])));
+        out[t * out_stride + h * vdim + d] = from_float<T>(o[d] * scale * norm_w[d] * gt);
+    }
+}
+
+// proj: elements [tokens, 2 G D + H DV + H], rows `stride` apart.  decay_in: float [tokens, H D].  gate_in: elements
+// [tokens, H DV], rows gate_stride apart.  conv_w: elements [2 G D + H DV, taps].  dt_bias float [H D], a_log float [H],
+// norm_w float [DV].  conv_state float [slots, 2 G D + H DV, taps - 1], s_state float [slots, H, D, DV]: a request's
+// rows by state_slots, taken as zero where seq_starts is 0.  scratch: float [tokens * (2 G D + 2 H DV + H D + H)].
+// The step's requests by cu_seqlens_q [seqs + 1]; token_seq [tokens].  out: elements [tokens, H DV].
+NVA_EXPORT int NVA_NAME(nva_channel_delta)(const void* proj, int64_t stride, const float* decay_in, const void* gate_in,
+                                           int64_t gate_stride, float* scratch, void* out, int64_t out_stride,
+                                           float* s_state, float* conv_state, const int32_t* token_seq,
+                                           const int32_t* cu_seqlens_q, const int32_t* seq_starts,
+                                           const int32_t* state_slots, int64_t seqs, int64_t tokens, int heads,
+                                           int kv_heads, int dim, int vdim, int taps, const void* conv_w,
+                                           const float* dt_bias, const float* a_log, const float* norm_w, float eps,
+                                           hipStream_t stream) {
+    if (tokens == 0) return 0;
+    if (tokens < 0 || tokens > 0x7fffffff || seqs <= 0 || seqs > 65535 * 32)
+        return nva_fail("channel_delta: bad counts tokens=%lld requests=%lld", (long long)tokens, (long long)seqs);
+    if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || heads > 65535 || dim <= 0 || vdim <= 0)
+        return nva_fail("channel_delta: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d", heads, kv_heads, dim, vdim);
+    if (dim > 256) return nva_fail("channel_delta: a head of %d key channels (up to 256)", dim);
+    if (taps < 1 || taps > DELTA_MAX_TAPS) return nva_fail("channel_delta: %d taps (1 to %d)", taps, DELTA_MAX_TAPS);
+    const int qk = kv_heads * dim, vv = heads * vdim, channels = 2 * qk + vv;
+    if (!proj || stride < channels + heads || !decay_in || !gate_in || gate_stride < vv || !scratch || !out || out_stride < vv ||
+        !s_state || (taps > 1 && !conv_state) || !token_seq || !cu_seqlens_q || !seq_starts || !state_slots || !conv_w ||
+        !dt_bias || !a_log || !norm_w)
+        return nva_fail("channel_delta: a tensor is missing or too narrow");
+    if (2 * (size_t)qk * sizeof(float) > 60 * 1024) return nva_fail("channel_delta: %d query and key channels do not fit the LDS", 2 * qk);
+    float* qn = scratch;
+    float* kn = qn + tokens * qk;
+    float* vf = kn + tokens * qk;
+    float* o_raw = vf + tokens * vv;
+    float* decay = o_raw + tokens * vv;
+    float* beta = decay + tokens * (int64_t)heads * dim;
+    {
+        auto kernel = delta_prepare_kernel<elem_t>;
+        const size_t lds = 2 * (size_t)qk * sizeof(float);
+        static bool raised = false;
+        if (!raised && lds > 48 * 1024) {
+            if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024) != hipSuccess)
+                return nva_fail("channel_delta: cannot have %zu bytes of LDS", lds);
+            raised = true;
+        }
+        hipLaunchKernelGGL(kernel, dim3((unsigned)tokens), dim3(256), lds, stream, (const elem_t*)proj, stride, decay_in,
+                           (const elem_t*)conv_w, dt_bias, a_log, conv_state, token_seq, cu_seqlens_q, seq_starts, state_slots,
+                           heads, kv_heads, dim, vdim, taps, qn, kn, vf, decay, beta);
+    }
+    if (taps > 1) {
+        if (seqs > 65535) return nva_fail("channel_delta: %lld requests a step", (long long)seqs);
+        hipLaunchKernelGGL(delta_keep_kernel<elem_t>, dim3((channels + 255) / 256, (unsigned)seqs), dim3(256), 0, stream,
+                           (const elem_t*)proj, stride, conv_state, cu_seqlens_q, seq_starts, state_slots, channels, taps);
+    }
+    {
+        const dim3 grid((unsigned)seqs, (unsigned)heads, (vdim + NVA_WAVE - 1) / NVA_WAVE);
+#define DELTA_SCAN(DM)                                                                                                   \
+        hipLaunchKernelGGL(delta_scan_kernel<DM>, grid, dim3(NVA_WAVE), 0, stream, qn, kn, vf, decay, beta, o_raw, s_state, \
+                           cu_seqlens_q, seq_starts, state_slots, heads, kv_heads, dim, vdim)
+        if (dim <= 32) DELTA_SCAN(32); else if (dim <= 64) DELTA_SCAN(64); else if (dim <= 128) DELTA_SCAN(128); else DELTA_SCAN(256);
+#undef DELTA_SCAN
+    }
+    hipLaunchKernelGGL(delta_finish_kernel<elem_t>, dim3((unsigned)tokens, (unsigned)heads), dim3(NVA_WAVE), 0, stream, o_raw,
+                       (const elem_t*)gate_in, gate_stride, norm_w, eps, (elem_t*)out, out_stride, heads, vdim);
+    return nva_check_launch("channel_delta");
+}
+
+NVA_DEFINE_LAST_ERROR(nva_delta)

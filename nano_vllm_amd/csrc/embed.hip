@@ -60,4 +60,31 @@ NVA_EXPORT int NVA_NAME(nva_scale_rows)(float* x, int64_t stride, int64_t rows, 
     return nva_check_launch("scale_rows");
 }
 
+// out[t] = float(table[ids[t]]) * factor: the start of a residual stream kept in float (an embedding with a
+// scale).  An id outside the table sets bit 0 of the flag and gives zeros.
+template <typename T>
+__global__ void __launch_bounds__(256)
+gather_scale_rows_kernel(const T* __restrict__ table, int64_t table_stride, int64_t table_rows, const int32_t* __restrict__ ids,
+                         float* __restrict__ out, int64_t out_stride, int width, float factor, int32_t* error_flag) {
+    const int64_t t = blockIdx.x;
+    const int id = ids[t];
+    const bool ok = id >= 0 && id < table_rows;
+    if (!ok && threadIdx.x == 0 && error_flag) atomicOr(error_flag, 1);
+    const T* src = table + (int64_t)(ok ? id : 0) * table_stride;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) out[t * out_stride + i] = ok ? to_float(src[i]) * factor : 0.f;
+}
+
+NVA_EXPORT int NVA_NAME(nva_gather_scale_rows)(const void* table, int64_t table_stride, int64_t table_rows, const int32_t* ids,
+                                               float* out, int64_t out_stride, int64_t count, int width, float factor,
+                                               int32_t* error_flag, hipStream_t stream) {
+    if (count == 0) return 0;
+    if (count < 0 || count > 0x7fffffff || width <= 0 || table_rows <= 0 || !table || !ids || !out || out_stride < width)
+        return nva_fail("gather_scale_rows: bad shape count=%lld width=%d rows=%lld", (long long)count, width,
+                        (long long)table_rows);
+    const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
+    hipLaunchKernelGGL(gather_scale_rows_kernel<elem_t>, dim3((unsigned)count), dim3(threads), 0, stream,
+                       (const elem_t*)table, table_stride, table_rows, ids, out, out_stride, width, factor, error_flag);
+    return nva_check_launch("gather_scale_rows");
+}
+
 NVA_DEFINE_LAST_ERROR(nva_embed)

@@ -7,10 +7,13 @@
 //             where a group holds one expert); the `group_keep` groups with the largest scores stay; of
 //             their experts the `top` with the largest scores are chosen (equal scores: the lower number);
 //             ids [tokens, top], weights [tokens, top] = scale * s.
+//             With softmax_top the logits (plus an optional float bias per expert) are compared as they are: the
+//             `top` largest are chosen (no groups) and weighted by the softmax over the chosen logits alone.
 //   plan      the pairs (token, choice) counted and sorted by expert: place[pair] = the pair's row among the
 //             sorted ones, rows[place] = pair; the sorted rows cut into tiles of 32 or 128 rows of one expert:
 //             tile_expert[i], tile_row0[i], tile_rows[i], and their number.
 //   up        h[row] = act(x[token of row] Wu_e^T)         rows sorted by expert, a tile of rows and 64 or 128
+//             gated: h[row] = act(x Wg_e^T) * (x Wu_e^T), an expert's matrix holding its gate rows, then its up rows
 //   down      o[row] = h[row] Wd_e^T                       outputs to a workgroup
 //   combine   y[token] = sum over its choices of weight * o[place] (+ add[token])
 //
@@ -39,7 +42,8 @@ __device__ __forceinline__ void moe_wave_best(float& v, int& idx) {
 // maximum over the wave.
 __global__ void __launch_bounds__(NVA_WAVE)
 moe_route_kernel(const float* __restrict__ logits, int64_t stride, int experts, int top, int group_count, int group_keep,
-                 float scale, int32_t* __restrict__ ids, float* __restrict__ weights) {
+                 float scale, int softmax_top, const float* __restrict__ bias, int32_t* __restrict__ ids,
+                 float* __restrict__ weights) {
     __shared__ float s_s[MOE_MAX_EXPERTS];
     __shared__ float g_s[MOE_MAX_EXPERTS];           // group scores; -inf once taken
     __shared__ unsigned char open_s[MOE_MAX_EXPERTS];
@@ -47,7 +51,8 @@ moe_route_kernel(const float* __restrict__ logits, int64_t stride, int experts, 
     const int lane = threadIdx.x;
     const bool all_groups = group_keep == group_count;
     for (int e = lane; e < experts; e += NVA_WAVE) {
-        s_s[e] = 1.f / (1.f + expf(-logits[t * stride + e]));
+        const float z = logits[t * stride + e] + (bias ? bias[e] : 0.f);
+        s_s[e] = softmax_top ? z : 1.f / (1.f + expf(-z));
         open_s[e] = all_groups ? 1 : 0;
     }
     __syncthreads();
@@ -84,9 +89,16 @@ moe_route_kernel(const float* __restrict__ logits, int64_t stride, int experts, 
         if (lane == 0) {
             open_s[best] = 0;
             ids[t * top + k] = best;
-            weights[t * top + k] = scale * v;
+            weights[t * top + k] = softmax_top ? v : scale * v;
         }
         __syncthreads();
+    }
+    if (softmax_top && lane == 0) {
+        // the chosen logits, largest first: their softmax among themselves, summed in the order of the choice
+        const float m = weights[t * top];
+        float sum = 0.f;
+        for (int k = 0; k < top; ++k) sum += expf(weights[t * top + k] - m);
+        for (int k = 0; k < top; ++k) weights[t * top + k] = expf(weights[t * top + k] - m) / sum;
     }
 }
 
@@ -131,7 +143,8 @@ moe_plan_kernel(const int32_t* __restrict__ ids, int64_t pairs, int experts, int
 
 // Tile product: out[row0 + r, n0 + c] = f(sum_k a[src(row0 + r), k] * w[e * n + n0 + c, k]).
 // UP: src = token of the pair (rows[row] / top), f = act; else src = the row itself, f = identity.
-template <typename T, bool UP>
+// GATED (with UP): the expert's matrix has 2 n rows, gate rows then up rows, and out = act(gate sum) * up sum.
+template <typename T, bool UP, bool GATED = false>
 __global__ void __launch_bounds__(256)
 moe_tile_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__ w, int n, int k,
                 const int32_t* __restrict__ rows, int top, const int32_t* __restrict__ tile_expert,
@@ -139,6 +152,7 @@ moe_tile_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__
                 const int32_t* __restrict__ num_tiles, int act, T* __restrict__ out, int64_t out_stride) {
     __shared__ float a_s[MOE_BM][MOE_BK + 1];
     __shared__ float w_s[MOE_BN][MOE_BK + 1];
+    __shared__ float u_s[GATED ? MOE_BN : 1][MOE_BK + 1];          // the up rows of the same outputs
     __shared__ int src_s[MOE_BM];
     const int tile = blockIdx.x;
     if (tile >= num_tiles[0]) return;
@@ -147,9 +161,10 @@ moe_tile_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__
     const int tid = threadIdx.x;
     if (tid < MOE_BM) src_s[tid] = tid < nrows ? (UP ? rows[row0 + tid] / top : row0 + tid) : -1;
     __syncthreads();
-    const T* we = w + (int64_t)e * n * k;
+    const T* we = w + (int64_t)e * (GATED ? 2 : 1) * n * k;
     const int ty = tid / 16, tx = tid % 16;          // rows ty, ty + 16; columns tx + 16 j
     float acc[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    float up[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
     for (int k0 = 0; k0 < k; k0 += MOE_BK) {
         for (int i = tid; i < MOE_BM * MOE_BK; i += 256) {
             const int r = i / MOE_BK, c = i % MOE_BK;
@@ -158,6 +173,7 @@ moe_tile_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__
         for (int i = tid; i < MOE_BN * MOE_BK; i += 256) {
             const int r = i / MOE_BK, c = i % MOE_BK;
             w_s[r][c] = n0 + r < n && k0 + c < k ? to_float(we[(int64_t)(n0 + r) * k + k0 + c]) : 0.f;
+            if (GATED) u_s[r][c] = n0 + r < n && k0 + c < k ? to_float(we[(int64_t)(n + n0 + r) * k + k0 + c]) : 0.f;
         }
         __syncthreads();
 #pragma unroll
@@ -168,6 +184,11 @@ moe_tile_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__
                 const float b = w_s[tx + 16 * j][c];
                 acc[0][j] += a0 * b;
                 acc[1][j] += a1 * b;
+                if (GATED) {
+                    const float u = u_s[tx + 16 * j][c];
+                    up[0][j] += a0 * u;
+                    up[1][j] += a1 * u;
+                }
             }
         }
         __syncthreads();
@@ -179,7 +200,9 @@ moe_tile_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int c = n0 + tx + 16 * j;
-            if (c < n) out[(int64_t)(row0 + r) * out_stride + c] = from_float<T>(UP ? nva_gate_act(act, acc[i][j]) : acc[i][j]);
+            if (c < n) out[(int64_t)(row0 + r) * out_stride + c] = from_float<T>(
+                GATED ? nva_gate_act(act, acc[i][j]) * up[i][j]
+                      : UP ? nva_gate_act(act, acc[i][j]) : acc[i][j]);
         }
     }
 }
@@ -190,12 +213,14 @@ moe_tile_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__
 // expert's matrix as the A operand of v_mfma_f32_16x16x32_bf16, straight from global memory into registers (a lane 16
 // bytes of a row a load; every byte of the matrix is read once per tile of rows), and all BM rows of x as B operands
 // from LDS, where the tile's rows are gathered a chunk of MOE_KC columns at a time.  A row's sum over k runs in the
-// order of the chunks whatever the tile it fell into.
+// order of the chunks whatever the tile it fell into.  GATED (with UP; WR a multiple of 32): the expert's matrix has
+// 2 n rows, gate rows then up rows; a wave takes WR / 2 outputs, the first half of its fragments their gate rows and
+// the second half their up rows, and gates in its epilogue.
 typedef __attribute__((ext_vector_type(8))) __bf16 moe_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float moe_f32x4;
 #define MOE_KC 128
 
-template <int BM, int WR, bool UP>
+template <int BM, int WR, bool UP, bool GATED = false>
 __global__ void __launch_bounds__(256)
 moe_mfma_kernel(const __bf16* __restrict__ a, int64_t a_stride, const __bf16* __restrict__ w, int n, int k,
                 const int32_t* __restrict__ rows, int top, const int32_t* __restrict__ tile_expert,
@@ -211,13 +236,17 @@ moe_mfma_kernel(const __bf16* __restrict__ a, int64_t a_stride, const __bf16* __
     if (tile >= num_tiles[0]) return;
     const int e = tile_expert[tile], row0 = tile_row0[tile], nrows = tile_rows[tile];
     const int tid = threadIdx.x, wave = tid / NVA_WAVE, lane = tid % NVA_WAVE, col = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.y * 4 * WR + wave * WR;
+    static_assert(!GATED || (UP && FR % 2 == 0), "gating needs an even number of fragments");
+    constexpr int WO = GATED ? WR / 2 : WR;                 // outputs of a wave
+    constexpr int FO = GATED ? FR / 2 : FR;                 // fragments of 16 outputs
+    const int n0 = blockIdx.y * 4 * WO + wave * WO;
     if (tid < BM) src_s[tid] = tid < nrows ? (UP ? rows[row0 + tid] / top : row0 + tid) : -1;
     __syncthreads();
-    const __bf16* we = w + (int64_t)e * n * k;
+    const __bf16* we = w + (int64_t)e * (GATED ? 2 : 1) * n * k;
     const __bf16* wrow[FR];
 #pragma unroll
-    for (int f = 0; f < FR; ++f) wrow[f] = we + (int64_t)min(n0 + 16 * f + col, n - 1) * k + 8 * g;
+    for (int f = 0; f < FR; ++f)
+        wrow[f] = we + ((int64_t)min(n0 + 16 * (f % FO) + col, n - 1) + (f >= FO ? n : 0)) * k + 8 * g;
     // the rows of x this thread gathers: piece i is row (tid + 256 i) / (MOE_KC / 8), columns 8 ((tid + 256 i) % (MOE_KC / 8))
     const __bf16* xsrc[XP];
     int xcol[XP];
@@ -280,9 +309,9 @@ moe_mfma_kernel(const __bf16* __restrict__ a, int64_t a_stride, const __bf16* __
         chunk(k0, fa0, fa1, x_s[0], x_s[1]);
         if (k0 + MOE_KC < k) chunk(k0 + MOE_KC, fa1, fa0, x_s[1], x_s[0]);
     }
-    // acc[f][b][i] = out[row 16 b + col][n0 + 16 f + 4 g + i]
+    // acc[f][b][i] = out[row 16 b + col][n0 + 16 f + 4 g + i]  (gated: fragment f + FO holds the up sums of the same outputs)
 #pragma unroll
-    for (int f = 0; f < FR; ++f)
+    for (int f = 0; f < FO; ++f)
 #pragma unroll
         for (int b = 0; b < MB; ++b) {
             const int r = 16 * b + col;
@@ -290,7 +319,10 @@ moe_mfma_kernel(const __bf16* __restrict__ a, int64_t a_stride, const __bf16* __
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int c = n0 + 16 * f + 4 * g + i;
-                if (c < n) out[(int64_t)(row0 + r) * out_stride + c] = (__bf16)(UP ? nva_gate_act(act, acc[f][b][i]) : acc[f][b][i]);
+                float v = acc[f][b][i];
+                if (GATED) v = nva_gate_act(act, v) * acc[GATED ? f + FO : f][b][i];
+                else if (UP) v = nva_gate_act(act, v);
+                if (c < n) out[(int64_t)(row0 + r) * out_stride + c] = (__bf16)v;
             }
         }
 }
@@ -311,8 +343,8 @@ moe_combine_kernel(const T* __restrict__ o, int64_t o_stride, const int32_t* __r
 }
 
 NVA_EXPORT int NVA_NAME(nva_moe_route)(const float* logits, int64_t stride, int64_t tokens, int experts, int top,
-                                       int group_count, int group_keep, float scale, int32_t* ids, float* weights,
-                                       hipStream_t stream) {
+                                       int group_count, int group_keep, float scale, int softmax_top, const float* bias,
+                                       int32_t* ids, float* weights, hipStream_t stream) {
     if (tokens == 0) return 0;
     if (tokens < 0 || tokens > 0x7fffffff || experts <= 0 || experts > MOE_MAX_EXPERTS)
         return nva_fail("moe_route: bad counts tokens=%lld experts=%d (up to %d)", (long long)tokens, experts, MOE_MAX_EXPERTS);
@@ -321,7 +353,7 @@ NVA_EXPORT int NVA_NAME(nva_moe_route)(const float* logits, int64_t stride, int6
         return nva_fail("moe_route: %d of %d experts in %d groups of which %d stay", top, experts, group_count, group_keep);
     if (!logits || !ids || !weights || stride < experts) return nva_fail("moe_route: a tensor is missing");
     hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)tokens), dim3(NVA_WAVE), 0, stream, logits, stride, experts, top,
-                       group_count, group_keep, scale, ids, weights);
+                       group_count, group_keep, scale, softmax_top ? 1 : 0, bias, ids, weights);
     return nva_check_launch("moe_route");
 }
 
@@ -335,12 +367,13 @@ static int moe_tile_rows(int64_t pairs, int experts, int k, int ff) {
 }
 NVA_EXPORT int NVA_NAME(nva_moe_tile_rows)(int64_t pairs, int experts, int k, int ff) { return moe_tile_rows(pairs, experts, k, ff); }
 
-// x [tokens, k] elements; ids, weights [tokens, top]; up [E * ff, k], down [E * k, ff] elements; add [tokens, k] or null.
+// x [tokens, k] elements; ids, weights [tokens, top]; up [E * ff, k] (gated: [E * 2 ff, k], an expert's gate rows, then
+// its up rows), down [E * k, ff] elements; add [tokens, k] or null.
 // Scratch: place, rows int32 [tokens * top]; tiles int32 [3 * max_tiles + 1] with max_tiles = tokens * top / MOE_BM + E
 // (expert, first row, rows of every tile, then their number); hidden [tokens * top, ff], outs [tokens * top, k] elements.
 NVA_EXPORT int NVA_NAME(nva_moe_experts)(const void* x, int64_t x_stride, const int32_t* ids, const float* weights,
                                          int64_t tokens, int top, int experts, int k, int ff, const void* up,
-                                         const void* down, int act, const void* add, int64_t add_stride, int32_t* place,
+                                         const void* down, int act, int gated, const void* add, int64_t add_stride, int32_t* place,
                                          int32_t* rows, int32_t* tiles, int64_t max_tiles, void* hidden, void* outs, void* y,
                                          int64_t y_stride, hipStream_t stream) {
     if (tokens == 0) return 0;
@@ -370,11 +403,26 @@ NVA_EXPORT int NVA_NAME(nva_moe_experts)(const void* x, int64_t x_stride, const 
         hipLaunchKernelGGL((moe_mfma_kernel<BMV, WRV, false>), dim3((unsigned)max_tiles, (k + 4 * WRV - 1) / (4 * WRV)),        \
                            dim3(256), 0, stream, (const __bf16*)hidden, (int64_t)ff, (const __bf16*)down, k, ff, rows, top,     \
                            tile_expert, tile_row0, tile_rows, num_tiles, act, (__bf16*)outs, (int64_t)k)
-        if (bm == 128) { MOE_LAUNCH(128, 32); } else { MOE_LAUNCH(32, 16); }
+#define MOE_LAUNCH_GATED(BMV, WRV)                                                                                            \
+        hipLaunchKernelGGL((moe_mfma_kernel<BMV, WRV, true, true>), dim3((unsigned)max_tiles, (ff + 2 * WRV - 1) / (2 * WRV)),  \
+                           dim3(256), 0, stream, (const __bf16*)x, x_stride, (const __bf16*)up, ff, k, rows, top, tile_expert, \
+                           tile_row0, tile_rows, num_tiles, act, (__bf16*)hidden, (int64_t)ff);                                 \
+        hipLaunchKernelGGL((moe_mfma_kernel<BMV, WRV / 2, false>), dim3((unsigned)max_tiles, (k + 2 * WRV - 1) / (2 * WRV)),    \
+                           dim3(256), 0, stream, (const __bf16*)hidden, (int64_t)ff, (const __bf16*)down, k, ff, rows, top,     \
+                           tile_expert, tile_row0, tile_rows, num_tiles, act, (__bf16*)outs, (int64_t)k)
+        if (gated) {
+            if (bm == 128) { MOE_LAUNCH_GATED(128, 64); } else { MOE_LAUNCH_GATED(32, 32); }
+        } else if (bm == 128) { MOE_LAUNCH(128, 32); } else { MOE_LAUNCH(32, 16); }
+#undef MOE_LAUNCH_GATED
 #undef MOE_LAUNCH
     } else
 #endif
     {
+    if (gated)
+        hipLaunchKernelGGL((moe_tile_kernel<elem_t, true, true>), dim3((unsigned)max_tiles, (ff + MOE_BN - 1) / MOE_BN), dim3(256), 0,
+                           stream, (const elem_t*)x, x_stride, (const elem_t*)up, ff, k, rows, top, tile_expert, tile_row0,
+                           tile_rows, num_tiles, act, (elem_t*)hidden, (int64_t)ff);
+    else
     hipLaunchKernelGGL((moe_tile_kernel<elem_t, true>), dim3((unsigned)max_tiles, (ff + MOE_BN - 1) / MOE_BN), dim3(256), 0,
                        stream, (const elem_t*)x, x_stride, (const elem_t*)up, ff, k, rows, top, tile_expert, tile_row0,
                        tile_rows, num_tiles, act, (elem_t*)hidden, (int64_t)ff);

@@ -248,6 +248,76 @@ NVA_EXPORT int NVA_NAME(nva_stream_rms_norm)(const void* a, int64_t a_stride, co
     return nva_check_launch("stream_rms_norm");
 }
 
+// ---------------------------------------------------------------------------- a normed addend into the float stream
+// A sublayer's output enters the stream through a norm of its own and a constant, and the stream is normed
+// for the next sublayer, all in one pass over the row:
+//     u = a / sqrt(mean(a^2) + eps_a) * wa            a elements, or a split product's partial sums
+//     r <- r + mult * u
+//     y = r / sqrt(mean(r^2) + eps) * w               rounded once, to the element type
+// All arithmetic in float; r float, in place.  One workgroup a row, which keeps its entries between the sums.
+template <typename T>
+__global__ void __launch_bounds__(1024)
+stream_post_norm_kernel(const T* __restrict__ a, int64_t a_stride, PartialInput pa, const void* __restrict__ a_weight,
+                        int aw_is_f32, float a_eps, float mult, float* residual, int64_t r_stride,
+                        const void* __restrict__ weight, int w_is_f32, T* __restrict__ y, int64_t y_stride, int width,
+                        float eps) {
+    __shared__ float scratch[16];
+    const int64_t row = blockIdx.x;
+    const T* ar = a ? a + row * a_stride : nullptr;
+    float* rr = residual + row * r_stride;
+    T* yr = y + row * y_stride;
+    constexpr int KEEP = 8;                       // entries a thread keeps between the passes
+    float kept[KEEP];
+    float ss = 0.f;
+    int n = 0;
+    for (int i = threadIdx.x; i < width; i += blockDim.x, ++n) {
+        const float v = pa.sums ? partial_value<T>(pa, row, width, i) : to_float(ar[i]);
+        if (n < KEEP) kept[n] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float a_scale = rsqrtf(ss / (float)width + a_eps) * mult;
+    float ss2 = 0.f;
+    n = 0;
+    for (int i = threadIdx.x; i < width; i += blockDim.x, ++n) {
+        const float v = n < KEEP ? kept[n] : (pa.sums ? partial_value<T>(pa, row, width, i) : to_float(ar[i]));
+        const float wa = aw_is_f32 ? static_cast<const float*>(a_weight)[i] : to_float(static_cast<const T*>(a_weight)[i]);
+        const float s = rr[i] + v * a_scale * wa;
+        rr[i] = s;
+        if (n < KEEP) kept[n] = s;
+        ss2 += s * s;
+    }
+    ss2 = block_sum(ss2, scratch);
+    const float scale = rsqrtf(ss2 / (float)width + eps);
+    n = 0;
+    for (int i = threadIdx.x; i < width; i += blockDim.x, ++n) {
+        const float s = n < KEEP ? kept[n] : rr[i];
+        const float w = w_is_f32 ? static_cast<const float*>(weight)[i] : to_float(static_cast<const T*>(weight)[i]);
+        yr[i] = from_float<T>(s * scale * w);
+    }
+}
+
+// a: elements [rows, width], or (a_sums) partial sums [splits][rows][width] with an optional bias.
+NVA_EXPORT int NVA_NAME(nva_stream_post_norm)(const void* a, int64_t a_stride, const float* a_sums, int a_splits,
+                                              int64_t a_split_stride, const void* a_bias, const void* a_weight,
+                                              int aw_is_f32, float a_eps, float mult, float* residual, int64_t r_stride,
+                                              const void* weight, int w_is_f32, void* y, int64_t y_stride, int64_t rows,
+                                              int width, float eps, hipStream_t stream) {
+    if (rows == 0) return 0;
+    if (rows < 0 || rows > 0x7fffffff || width <= 0)
+        return nva_fail("stream_post_norm: bad shape rows=%lld width=%d", (long long)rows, width);
+    if (!residual || !y || !weight || !a_weight || (!a && !a_sums))
+        return nva_fail("stream_post_norm: the addend, its weight, the stream, the weight and the output are needed");
+    if (a_sums && (a_splits <= 0 || a_split_stride < rows * (int64_t)width)) return nva_fail("stream_post_norm: bad partial sums");
+    const PartialInput pa{a_sums, a_splits, a_split_stride, a_bias};
+    const int threads = a_sums && rows <= 64 && width >= 1024 ? 1024
+                        : width >= 2048 ? 512 : width >= 1024 ? 256 : width >= 256 ? 128 : 64;
+    hipLaunchKernelGGL((stream_post_norm_kernel<elem_t>), dim3((unsigned)rows), dim3(threads), 0, stream,
+                       (const elem_t*)a, a_stride, pa, a_weight, aw_is_f32, a_eps, mult, residual, r_stride, weight, w_is_f32,
+                       (elem_t*)y, y_stride, width, eps);
+    return nva_check_launch("stream_post_norm");
+}
+
 // ---------------------------------------------------------------------------- Dynamic Tanh on the float stream
 //     r <- r + a + b   (first: r <- a + b)        a, b elements or absent
 //     y = tanh(alpha * r) * w + c                  alpha one float read on the device, w and c float vectors

@@ -15,6 +15,8 @@
 // are float; q is written out and k, v into the cache, each rounded once to the element type.  The weights are
 // plain (not one-plus), stored as elements or float.
 // Cache layout: K [pages, Hkv, page, D], V [pages, Hkv, page / vt, DV, vt] (common.h).
+// With per_head the two norms run over every head by itself, mean over its D entries, with weights of D
+// entries that the heads share.
 // One workgroup per token.
 #include "common.h"
 
@@ -26,8 +28,8 @@ qk_rownorm_store_kernel(const T* __restrict__ qkv, int64_t stride, PartialInput 
                         const int32_t* __restrict__ positions, float temp_coef, int temp_every,
                         const float* __restrict__ rot_table, int rot,
                         const int32_t* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                        int page_size) {
-    extern __shared__ __attribute__((aligned(16))) float row_s[];      // the token's row, as float
+                        int page_size, int per_head) {
+    extern __shared__ __attribute__((aligned(16))) float row_s[];      // the token's row, as float; then a scale per head
     __shared__ float scratch[16];
     const int64_t t = blockIdx.x;
     const int qd = num_heads * head_dim, kd = num_kv_heads * head_dim, vd = num_kv_heads * v_dim;
@@ -43,10 +45,23 @@ qk_rownorm_store_kernel(const T* __restrict__ qkv, int64_t stride, PartialInput 
         row_s[i] = x;
         if (i < qd) sq += x * x; else if (i < qd + kd) sk += x * x;
     }
-    sq = block_sum(sq, scratch);
-    sk = kd ? block_sum(sk, scratch) : 0.f;
+    float* const head_scale = row_s + width;                           // [num_heads + num_kv_heads], with per_head
+    if (per_head) {
+        __syncthreads();
+        const int wave = tid / NVA_WAVE, lane = tid % NVA_WAVE, nwaves = blockDim.x / NVA_WAVE;
+        for (int hh = wave; hh < num_heads + num_kv_heads; hh += nwaves) {
+            float ss = 0.f;
+            for (int d = lane; d < head_dim; d += NVA_WAVE) ss += row_s[hh * head_dim + d] * row_s[hh * head_dim + d];
+            ss = wave_sum(ss);
+            if (lane == 0) head_scale[hh] = rsqrtf(ss / (float)head_dim + eps);
+        }
+        __syncthreads();
+    } else {
+        sq = block_sum(sq, scratch);
+        sk = kd ? block_sum(sk, scratch) : 0.f;
+    }
 
-    float q_scale = q_weight ? rsqrtf(sq / (float)qd + eps) : 1.f;
+    float q_scale = q_weight && !per_head ? rsqrtf(sq / (float)qd + eps) : 1.f;
     if (temp_coef != 0.f) q_scale *= 1.f + temp_coef * logf((float)steps + 1.f);
     T* qrow = q_out + t * q_stride;
     const float* rot_row = rot_table ? rot_table + t * (int64_t)rot : nullptr;
@@ -56,18 +71,19 @@ qk_rownorm_store_kernel(const T* __restrict__ qkv, int64_t stride, PartialInput 
     };
     // entry i of a projection that starts at `at` in the row, scaled and weighted, then turned with its partner
     auto prepared = [&](int at, int i, float scale, const void* w) -> float {
-        const float x = row_s[at + i] * scale * weight_of(w, i);
         const int d = i % head_dim;
+        if (per_head && w) scale *= head_scale[(at + i) / head_dim];   // (at is a multiple of the head size)
+        const float x = row_s[at + i] * scale * weight_of(w, per_head ? d : i);
         if (!rot_row || d >= rot) return x;
         const int f = d < half ? d : d - half;
         const int j = d < half ? i + half : i - half;
-        const float y = row_s[at + j] * scale * weight_of(w, j);
+        const float y = row_s[at + j] * scale * weight_of(w, per_head ? j % head_dim : j);
         const float c = rot_row[f], sn = rot_row[half + f];
         return d < half ? x * c - y * sn : x * c + y * sn;
     };
     for (int i = tid; i < qd; i += blockDim.x) qrow[i] = from_float<T>(prepared(0, i, q_scale, q_weight));
     if (!kd || slot < 0 || !k_cache) return;
-    const float k_scale = k_weight ? rsqrtf(sk / (float)kd + eps) : 1.f;
+    const float k_scale = k_weight && !per_head ? rsqrtf(sk / (float)kd + eps) : 1.f;
     const int page = slot / page_size, off = slot % page_size;
     const int vt = nva_v_tile(page_size);
     for (int i = tid; i < kd; i += blockDim.x) {
@@ -85,7 +101,7 @@ qk_rownorm_store_kernel(const T* __restrict__ qkv, int64_t stride, PartialInput 
 // qkv: [tokens, Hq * D + Hkv * D + Hkv * DV] with rows `stride` elements apart, or (sums != null) the float
 // partial sums [splits][tokens][width] of the projection with its bias, which are added up here.
 // q_out: [tokens, Hq * D] with rows q_stride apart (it may be qkv itself: q is then rewritten in place).
-// q_weight [Hq * D], k_weight [Hkv * D]: both or none.  positions are needed with a temperature.
+// q_weight [Hq * D], k_weight [Hkv * D] (per_head: both [D]): both or none.  positions are needed with a temperature.
 // rot_table: float [tokens, rot], a row per token of this call, or null.
 // slots (with the caches) may be null: nothing is stored then.  num_kv_heads 0: the row holds q only.
 NVA_EXPORT int NVA_NAME(nva_qk_rownorm_store)(const void* qkv, int64_t stride, const float* sums, int splits,
@@ -94,7 +110,8 @@ NVA_EXPORT int NVA_NAME(nva_qk_rownorm_store)(const void* qkv, int64_t stride, c
                                               int head_dim, int v_dim, const void* q_weight, const void* k_weight,
                                               int w_is_f32, float eps, const int32_t* positions, float temp_coef,
                                               int temp_every, const float* rot_table, int rot, const int32_t* slots,
-                                              void* k_cache, void* v_cache, int page_size, hipStream_t stream) {
+                                              void* k_cache, void* v_cache, int page_size, int per_head,
+                                              hipStream_t stream) {
     if (tokens == 0) return 0;
     if (tokens < 0 || tokens > 0x7fffffff) return nva_fail("qk_rownorm_store: bad token count %lld", (long long)tokens);
     if (num_heads <= 0 || num_kv_heads < 0 || head_dim <= 0 || v_dim <= 0)
@@ -115,7 +132,7 @@ NVA_EXPORT int NVA_NAME(nva_qk_rownorm_store)(const void* qkv, int64_t stride, c
     if ((k_cache || v_cache) && (!k_cache || !v_cache || !slots || page_size <= 0 || !num_kv_heads))
         return nva_fail("qk_rownorm_store: storing needs both caches, the slots and the page size");
     auto kernel = qk_rownorm_store_kernel<elem_t>;
-    const size_t lds = (size_t)width * sizeof(float);
+    const size_t lds = (size_t)(width + (per_head ? num_heads + num_kv_heads : 0)) * sizeof(float);
     static bool raised = false;
     if (!raised && lds > 48 * 1024) {
         if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
@@ -127,7 +144,8 @@ NVA_EXPORT int NVA_NAME(nva_qk_rownorm_store)(const void* qkv, int64_t stride, c
     const int threads = tokens <= 64 && width >= 2048 ? 1024 : 256;
     hipLaunchKernelGGL(kernel, dim3((unsigned)tokens), dim3(threads), lds, stream, (const elem_t*)qkv, stride, part,
                        (elem_t*)q_out, q_stride, num_heads, num_kv_heads, head_dim, v_dim, q_weight, k_weight, w_is_f32, eps,
-                       positions, temp_coef, temp_every, rot_table, rot_table ? rot : 0, slots, (elem_t*)k_cache, (elem_t*)v_cache, page_size);
+                       positions, temp_coef, temp_every, rot_table, rot_table ? rot : 0, slots, (elem_t*)k_cache, (elem_t*)v_cache, page_size,
+                       per_head ? 1 : 0);
     return nva_check_launch("qk_rownorm_store");
 }
 

@@ -40,6 +40,7 @@ MODULES: Dict[str, Tuple[str, Tuple[Optional[str], ...]]] = {
     "retention": ("retention.hip", ("bf16", "f32")),
     "ssd": ("ssd.hip", ("bf16", "f32")),
     "moe": ("moe.hip", ("bf16", "f32")),
+    "delta": ("delta.hip", ("bf16", "f32")),
 }
 
 _HEADERS = ("common.h",)

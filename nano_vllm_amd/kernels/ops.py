@@ -345,6 +345,16 @@ class HipKernels:
 
     gather_rows = embedding
 
+    def embedding_scaled(self, table: torch.Tensor, ids: torch.Tensor, scale: float) -> torch.Tensor:
+        """float32 out[t] = table[ids[t]] * scale: the start of a residual stream kept in float32."""
+        rows, width, stride = _rows2d(table, "embedding table")
+        n = ids.shape[0]
+        _i32(ids, n, "embedding ids")
+        out = torch.empty((n, width), dtype=torch.float32, device=table.device)
+        library.call("embed", _suffix(table), "nva_gather_scale_rows", _p(table), c_i64(stride), c_i64(rows), _p(ids),
+                     _p(out), c_i64(width), c_i64(n), c_i32(width), c_f32(float(scale)), _p(self.fault_flag), self._stream())
+        return out
+
     # ------------------------------------------------------------------ norms
     def _norm_weight(self, weight: torch.Tensor, width: int, x: torch.Tensor):
         if weight.dim() != 1 or weight.shape[0] != width or not weight.is_contiguous():
@@ -419,6 +429,11 @@ class HipKernels:
         sum of the addends), then y = residual * rsqrt(mean(residual^2) + eps) * (offset + weight),
         all in float and rounded once.  addends: up to two tensors of the element type [rows, width].
         Returns (y, residual)."""
+        if any(hasattr(a, "mult") for a in addends):
+            if len(addends) != 1 or residual is None or offset != 0.0:
+                raise KernelError("stream_rms_norm: an addend with a norm of its own comes alone, into a stream that exists, "
+                                  "and goes with a plain weight")
+            return self._stream_post_norm(addends[0], residual, weight, eps, out)
         # a product left as partial sums is added up here, while it is read; anything else is a tensor
         addends = [a if isinstance(a, SplitSum) and self.fuse_split_sums else _t(a) for a in addends]
         if len(addends) > 2 or (residual is None and not addends):
@@ -458,6 +473,32 @@ class HipKernels:
         library.call("norm", _suffix(out), "nva_stream_rms_norm", *args, _p(residual), c_i64(rs), c_i32(1 if first else 0),
                      _p(weight), c_i32(wf), c_f32(offset), _p(out), c_i64(os_), c_i64(rows), c_i32(width), c_f32(eps),
                      self._stream())
+        return out, residual
+
+    def _stream_post_norm(self, addend, residual: torch.Tensor, weight: torch.Tensor, eps: float,
+                          out: Optional[torch.Tensor] = None):
+        """residual <- residual + mult * a / sqrt(mean(a^2) + eps_a) * w_a, then the stream's own norm, in one pass;
+        `addend` carries a (elements, or a product left as partial sums), w_a, eps_a and mult."""
+        a = addend.x if isinstance(addend.x, SplitSum) and self.fuse_split_sums else _t(addend.x)
+        rows, width = a.shape
+        rrows, rw, rs = _rows2d(residual, "stream_rms_norm residual")
+        if (rrows, rw) != (rows, width) or residual.dtype != torch.float32:
+            raise KernelError("stream_rms_norm: the residual stream must be float32 of the addend's shape")
+        if out is None:
+            out = torch.empty((rows, width), dtype=a.dtype, device=residual.device)
+        orows, ow, os_ = _rows2d(out, "stream_rms_norm output")
+        if (orows, ow) != (rows, width) or out.dtype != a.dtype:
+            raise KernelError("stream_rms_norm: output does not match")
+        wf = self._norm_weight(weight, width, out)
+        awf = self._norm_weight(addend.weight, width, out)
+        if isinstance(a, SplitSum):
+            src = [None, c_i64(0), _p(a.sums), c_i32(a.splits), c_i64(rows * width), _p(a.bias)]
+        else:
+            _, _, as_ = _rows2d(a, "stream_rms_norm addend")
+            src = [_p(a), c_i64(as_), None, c_i32(0), c_i64(0), None]
+        library.call("norm", _suffix(out), "nva_stream_post_norm", *src, _p(addend.weight), c_i32(awf), c_f32(float(addend.eps)),
+                     c_f32(float(addend.mult)), _p(residual), c_i64(rs), _p(weight), c_i32(wf), _p(out), c_i64(os_), c_i64(rows),
+                     c_i32(width), c_f32(eps), self._stream())
         return out, residual
 
     def stream_dyt(self, addends, residual: Optional[torch.Tensor], weight: torch.Tensor, bias: torch.Tensor,
@@ -555,32 +596,41 @@ class HipKernels:
         return out
 
     # ------------------------------------------------------------------ routed feed-forward
-    def moe_route(self, logits: torch.Tensor, top: int, group_count: int, group_keep: int, scale: float):
+    def moe_route(self, logits: torch.Tensor, top: int, group_count: int, group_keep: int, scale: float,
+                  routing: str = "sigmoid_groups", bias: Optional[torch.Tensor] = None):
         """From the router's float32 logits [tokens, experts]: int32 [tokens, top] experts and float32
         [tokens, top] weights (scale * sigmoid score).  Experts form group_count groups of neighbours; a
         group's score is the sum of its two largest scores; only experts of the group_keep best groups are
-        chosen, the `top` with the largest scores."""
+        chosen, the `top` with the largest scores.  routing "softmax_top": the `top` largest logits (plus the
+        float32 bias [experts], if any) are chosen and weighted by the softmax over the chosen alone."""
         rows, experts, ls = _rows2d(logits, "router logits")
         if logits.dtype != torch.float32:
             raise KernelError("moe_route: the logits must be float32")
+        if routing not in ("sigmoid_groups", "softmax_top"):
+            raise KernelError(f"moe_route: unknown routing {routing!r}")
+        if bias is not None and (bias.dtype != torch.float32 or tuple(bias.shape) != (experts,) or not bias.is_contiguous()):
+            raise KernelError(f"moe_route: the bias must be contiguous float32 [{experts}]")
         ids = torch.empty((rows, top), dtype=torch.int32, device=logits.device)
         weights = torch.empty((rows, top), dtype=torch.float32, device=logits.device)
         library.call("moe", self.suffix, "nva_moe_route", _p(logits), c_i64(ls), c_i64(rows), c_i32(experts), c_i32(top),
-                     c_i32(group_count), c_i32(group_keep), c_f32(scale), _p(ids), _p(weights), self._stream())
+                     c_i32(group_count), c_i32(group_keep), c_f32(scale), c_i32(1 if routing == "softmax_top" else 0),
+                     _p(bias), _p(ids), _p(weights), self._stream())
         return ids, weights
 
     def moe_experts(self, x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, up: torch.Tensor, down: torch.Tensor,
-                    num_experts: int, act: str = "relu2", add=None) -> torch.Tensor:
+                    num_experts: int, act: str = "relu2", add=None, gated: bool = False) -> torch.Tensor:
         """y[t] = sum over the choices c of weights[t, c] * act(x[t] Wu_e^T) Wd_e^T with e = ids[t, c] (+ add[t]).
-        up [E * ff, k] and down [E * k, ff] hold the experts' matrices one below the other."""
+        up [E * ff, k] and down [E * k, ff] hold the experts' matrices one below the other.  gated: up is
+        [E * 2 ff, k], an expert's gate rows and then its up rows, and the hidden layer act(x Wg_e^T) * (x Wu_e^T)."""
         if act not in self.PLAIN_ACTIVATIONS:
             raise KernelError(f"moe_experts: unknown activation {act!r}")
         x = _t(x)
         tokens, k, xs = _rows2d(x, "moe input")
-        if up.dim() != 2 or down.dim() != 2 or up.shape[0] % num_experts or up.shape[1] != k or not up.is_contiguous() \
+        per = num_experts * (2 if gated else 1)
+        if up.dim() != 2 or down.dim() != 2 or up.shape[0] % per or up.shape[1] != k or not up.is_contiguous() \
                 or not down.is_contiguous() or up.dtype != x.dtype or down.dtype != x.dtype:
             raise KernelError("moe_experts: the experts' matrices do not fit the input")
-        ff = up.shape[0] // num_experts
+        ff = up.shape[0] // per
         if tuple(down.shape) != (num_experts * k, ff):
             raise KernelError(f"moe_experts: down must be [{num_experts * k}, {ff}], got {tuple(down.shape)}")
         top = ids.shape[1] if ids.dim() == 2 else 0
@@ -602,8 +652,8 @@ class HipKernels:
         outs = torch.empty((pairs, k), dtype=x.dtype, device=x.device)
         y = torch.empty((tokens, k), dtype=x.dtype, device=x.device)
         library.call("moe", _suffix(x), "nva_moe_experts", _p(x), c_i64(xs), _p(ids), _p(weights), c_i64(tokens), c_i32(top),
-                     c_i32(num_experts), c_i32(k), c_i32(ff), _p(up), _p(down), c_i32(self.PLAIN_ACTIVATIONS[act]), _p(add),
-                     c_i64(add_stride), _p(ints[:pairs]), _p(ints[pairs:2 * pairs]), _p(ints[2 * pairs:]), c_i64(max_tiles),
+                     c_i32(num_experts), c_i32(k), c_i32(ff), _p(up), _p(down), c_i32(self.PLAIN_ACTIVATIONS[act]),
+                     c_i32(1 if gated else 0), _p(add), c_i64(add_stride), _p(ints[:pairs]), _p(ints[pairs:2 * pairs]), _p(ints[2 * pairs:]), c_i64(max_tiles),
                      _p(hidden), _p(outs), _p(y), c_i64(k), self._stream())
         return y
 
@@ -1097,8 +1147,10 @@ class HipKernels:
                          q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
                          positions: Optional[torch.Tensor], temp_coef: float, temp_every: int,
                          slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
-                         v_cache: Optional[torch.Tensor], rot_table: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """rot_table, float32 [tokens, rot]: after norm and temperature the first rot channels of every head
+                         v_cache: Optional[torch.Tensor], rot_table: Optional[torch.Tensor] = None,
+                         norm_per_head: bool = False) -> torch.Tensor:
+        """norm_per_head: the two norms run over every head by itself, with weights [head_dim] that the heads share.
+        rot_table, float32 [tokens, rot]: after norm and temperature the first rot channels of every head
         of q and k are rotated in pairs (i, i + rot / 2) by the token's row (rot / 2 cosines, then sines).
         q and k normed over the whole projection (all heads at once, plain weights [heads * head_dim]
         and [kv_heads * head_dim]), q scaled by the temperature 1 + temp_coef * ln(floor((p + 1) /
@@ -1116,7 +1168,7 @@ class HipKernels:
         wf = 0
         for w, n in ((q_weight, num_heads * head_dim), (k_weight, num_kv_heads * head_dim)):
             if w is not None:
-                wf = self._norm_weight(w, n, qkv)
+                wf = self._norm_weight(w, head_dim if norm_per_head else n, qkv)
         if num_kv_heads and (q_weight is None) != (k_weight is None):
             raise KernelError("qk norm: give both weights or none")
         if q_weight is not None and k_weight is not None and q_weight.dtype != k_weight.dtype:
@@ -1147,8 +1199,24 @@ class HipKernels:
         library.call("qk_rownorm", "bf16" if partial else _suffix(qkv), "nva_qk_rownorm_store", *source, c_i64(tokens),
                      c_i32(num_heads), c_i32(num_kv_heads), c_i32(head_dim), c_i32(v_head_dim), _p(q_weight), _p(k_weight),
                      c_i32(wf), c_f32(eps), _p(positions), c_f32(float(temp_coef)), c_i32(int(temp_every) if temp_coef else 1),
-                     _p(rot_table), c_i32(rot), _p(slots), _p(k_cache), _p(v_cache), c_i32(page_size), self._stream())
+                     _p(rot_table), c_i32(rot), _p(slots), _p(k_cache), _p(v_cache), c_i32(page_size),
+                     c_i32(1 if norm_per_head and q_weight is not None else 0), self._stream())
         return q
+
+    def sigmoid_mul(self, x: torch.Tensor, gate: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """x * sigmoid(gate), entry by entry, in float and rounded once; in place unless out is given."""
+        x, gate = _t(x), _t(gate)
+        rows, width, xs = _rows2d(x, "sigmoid_mul input")
+        grows, gw, gs = _rows2d(gate, "sigmoid_mul gate")
+        if (grows, gw) != (rows, width) or gate.dtype != x.dtype:
+            raise KernelError("sigmoid_mul: the gate does not match the input")
+        out = x if out is None else out
+        orows, ow, os_ = _rows2d(out, "sigmoid_mul output")
+        if (orows, ow) != (rows, width) or out.dtype != x.dtype:
+            raise KernelError("sigmoid_mul: output does not match the input")
+        library.call("activation", _suffix(x), "nva_sigmoid_mul", _p(x), c_i64(xs), _p(gate), c_i64(gs), _p(out), c_i64(os_),
+                     c_i64(rows), c_i32(width), self._stream())
+        return out
 
     @staticmethod
     def _check_cache(k_cache, v_cache, num_kv_heads, head_dim, dtype, v_head_dim=None) -> int:
@@ -1169,8 +1237,10 @@ class HipKernels:
                         k_cache: torch.Tensor, v_cache: torch.Tensor, batch, group: int, scale: float,
                         window: Optional[int] = None, out: Optional[torch.Tensor] = None,
                         v_head_dim: Optional[int] = None, sinks: Optional[torch.Tensor] = None,
-                        chunk: Optional[int] = None) -> torch.Tensor:
+                        chunk: Optional[int] = None, softcap: Optional[float] = None, keep_first: int = 0) -> torch.Tensor:
         """chunk: a query at position p reads the keys from floor(p / chunk) * chunk on only.
+        softcap: a score s (after the scale) becomes softcap * tanh(s / softcap).  keep_first (with a window):
+        every query also reads the first keep_first positions of its sequence, however far back.
         Causal attention of the step's tokens over the cache.  `batch` is the step's
         StepBatch; `group` selects its block tables.  q [T, heads*head_dim] (rows may be strided).
         v_head_dim: the size of a head's values where it is not head_dim (the output is then
@@ -1205,7 +1275,12 @@ class HipKernels:
         # them where its shape limits allow; everything else runs the general kernel
         start = 0
         # (the matrix-core kernels fold the scale into the exponent, which needs it positive)
-        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and v_dim == head_dim
+        cap = float(softcap) if softcap else 0.0
+        keep = int(keep_first) if window and keep_first else 0
+        if cap < 0.0 or keep < 0:
+            raise KernelError("attention: a negative softcap or number of kept positions")
+        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and v_dim == head_dim \
+            and cap == 0.0 and keep == 0
         if batch.num_decode > 0 and mfma and \
                 self._decode_kernel_takes(num_heads // num_kv_heads, head_dim, page_size, q, qs, out, os_):
             start = batch.num_decode
@@ -1229,8 +1304,8 @@ class HipKernels:
             library.call("attn_generic", _suffix(q), "nva_paged_attention_tiled", _p(q), c_i64(qs), _p(out), c_i64(os_),
                          _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.cu_seqlens_q),
                          _p(batch.kv_lens), _p(tiles), c_i64(tiles.shape[0]), c_i32(num_heads), c_i32(num_kv_heads),
-                         c_i32(head_dim), c_i32(v_dim), c_i32(page_size), c_f32(scale), c_i32(chunk or 0), _p(sinks),
-                         _p(self.fault_flag), self._stream())
+                         c_i32(head_dim), c_i32(v_dim), c_i32(page_size), c_f32(scale), c_i32(chunk or 0), c_f32(cap),
+                         _p(sinks), _p(self.fault_flag), self._stream())
             tokens = batch.num_decode            # what is left: the single tokens before the portions
         if start < tokens:
             n = tokens - start
@@ -1238,7 +1313,63 @@ class HipKernels:
                          _p(out[start:]), c_i64(os_), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
                          _p(batch.token_seq[start:]), _p(batch.positions[start:]), c_i64(n), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(v_dim), c_i32(page_size), c_f32(scale),
-                         c_i32(window or 0), c_i32(chunk or 0), _p(sinks), _p(self.fault_flag), self._stream())
+                         c_i32(window or 0), c_i32(chunk or 0), c_i32(keep), c_f32(cap), _p(sinks), _p(self.fault_flag),
+                         self._stream())
+        return out
+
+    # ------------------------------------------------------------------ delta rule
+    def channel_delta(self, proj: torch.Tensor, decay_in: torch.Tensor, gate_in: torch.Tensor, heads: int, kv_heads: int,
+                      dim: int, vdim: int, taps: int, conv_w: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor,
+                      norm_w: torch.Tensor, eps: float, conv_state: torch.Tensor, s_state: torch.Tensor, batch,
+                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The gated delta rule with a decay per key channel over the step's tokens: proj [T, 2 G D + H DV + H] =
+        [q | k | v | b] with G = kv_heads heads of D = dim and H = heads heads of DV = vdim.  q, k, v pass a causal
+        convolution of `taps` taps per channel (conv_w [C, taps]) and silu; q and k become unit vectors per head (q
+        times D^-1/2); beta = sigmoid(b); a = exp(-exp(a_log) * softplus(decay_in + dt_bias)), decay_in float32
+        [T, H D]; per head S <- diag(a) S, u = beta (v - S^T k), S <- S + k u^T, o = S^T q; then o's RMS norm per head
+        times norm_w [DV] times sigmoid(gate_in), gate_in [T, H DV].  s_state float32 [slots, H, D, DV] and conv_state
+        float32 [slots, C, taps - 1] hold a request's state in the row batch.state_slots names, taken as zero where
+        batch.seq_starts is 0.  Returns [T, H DV] of proj's type."""
+        proj, gate_in = _t(proj), _t(gate_in)
+        decay_in = _t(decay_in)
+        tokens, width, stride = _rows2d(proj, "delta-rule projections")
+        qk, vv, hd = kv_heads * dim, heads * vdim, heads * dim
+        channels = 2 * qk + vv
+        if width != channels + heads:
+            raise KernelError(f"channel_delta: projections of width {width}, expected {channels + heads}")
+        if decay_in.dtype != torch.float32 or tuple(decay_in.shape) != (tokens, hd) or not decay_in.is_contiguous():
+            raise KernelError(f"channel_delta: the decay's input must be contiguous float32 [{tokens}, {hd}]")
+        grows, gw, gs = _rows2d(gate_in, "delta-rule gate")
+        if (grows, gw) != (tokens, vv) or gate_in.dtype != proj.dtype:
+            raise KernelError("channel_delta: the gate's input does not match")
+        if s_state.dtype != torch.float32 or tuple(s_state.shape[1:]) != (heads, dim, vdim) or not s_state.is_contiguous():
+            raise KernelError(f"channel_delta: the state must be contiguous float32 [slots, {heads}, {dim}, {vdim}]")
+        if conv_state.dtype != torch.float32 or tuple(conv_state.shape) != (s_state.shape[0], channels, taps - 1) or \
+                not conv_state.is_contiguous():
+            raise KernelError(f"channel_delta: the kept inputs must be contiguous float32 [slots, {channels}, {taps - 1}]")
+        if tuple(conv_w.shape) != (channels, taps) or conv_w.dtype != proj.dtype or not conv_w.is_contiguous():
+            raise KernelError("channel_delta: the convolution's weights do not fit")
+        for v, n, what in ((dt_bias, hd, "dt_bias"), (a_log, heads, "a_log"), (norm_w, vdim, "norm_w")):
+            if v.dtype != torch.float32 or tuple(v.shape) != (n,) or not v.is_contiguous():
+                raise KernelError(f"channel_delta: {what} must be contiguous float32 [{n}]")
+        seqs = batch.num_seqs
+        _i32(batch.token_seq, tokens, "token_seq")
+        _i32(batch.cu_seqlens_q, seqs + 1, "cu_seqlens_q")
+        _i32(batch.seq_starts, seqs, "seq_starts")
+        _i32(batch.state_slots, seqs, "state_slots")
+        if sum(batch.q_lens) != tokens:
+            raise KernelError("channel_delta: the batch does not describe the projections' rows")
+        if out is None:
+            out = torch.empty((tokens, vv), dtype=proj.dtype, device=proj.device)
+        orows, ow, os_ = _rows2d(out, "delta-rule output")
+        if (orows, ow) != (tokens, vv) or out.dtype != proj.dtype:
+            raise KernelError("channel_delta: output does not match")
+        scratch = torch.empty(tokens * (2 * qk + 2 * vv + hd + heads), dtype=torch.float32, device=proj.device)
+        library.call("delta", _suffix(proj), "nva_channel_delta", _p(proj), c_i64(stride), _p(decay_in), _p(gate_in), c_i64(gs),
+                     _p(scratch), _p(out), c_i64(os_), _p(s_state), _p(conv_state if taps > 1 else None), _p(batch.token_seq),
+                     _p(batch.cu_seqlens_q), _p(batch.seq_starts), _p(batch.state_slots), c_i64(seqs), c_i64(tokens),
+                     c_i32(heads), c_i32(kv_heads), c_i32(dim), c_i32(vdim), c_i32(taps), _p(conv_w), _p(dt_bias), _p(a_log),
+                     _p(norm_w), c_f32(eps), self._stream())
         return out
 
     # ------------------------------------------------------------------ state-space layer

@@ -319,7 +319,7 @@ def test_another_embedding_and_head_are_registered_not_edited_in(tmp_path):
         def on_weights_loaded(self):                  # called once, after every parameter is there
             assert self.weights["weight"].shape == (384, 96)
             type(self).told += 1
-            self.factor = torch.tensor(float(self.params["scale"]))
+            self.factor = torch.tensor(float(self.params["toy_scale"]))
 
         def forward(self, ids):
             return super().forward(ids) * self.factor
@@ -332,7 +332,7 @@ def test_another_embedding_and_head_are_registered_not_edited_in(tmp_path):
     def toy_spec(cfg):
         s = build_spec(cfg)
         return dataclasses.replace(
-            s, embedding=PartSpec("toy_scaled_embedding", {**s.embedding.params, "scale": scale}),
+            s, embedding=PartSpec("toy_scaled_embedding", {**s.embedding.params, "toy_scale": scale}),
             head=PartSpec("toy_capped_head", {**s.head.params, "cap": cap}))
 
     register_part("embedding", "toy_scaled_embedding", ScaledEmbedding, replace=True)
