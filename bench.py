@@ -30,6 +30,12 @@ with both designs' numbers per size.
 does the same for the Mafarax design (every layer a chunked attention and a state-space layer side by
 side, and a routed feed-forward whose experts a token runs add up to the dense layer's inner size),
 beside Nozurax and Qwen3 at equal layer sizes.
+
+    python bench.py --design kirisun [--design-sizes 1024,2048,4096] [--layers 4]
+
+does the same for the Kirisun design (layers of the channel-wise delta rule and of a gated window attention in
+turn, each with a routed feed-forward of gated experts whose chosen experts add up to the dense layer's inner
+size), beside Mafarax and Qwen3 at equal layer sizes.
 """
 import argparse
 import json
@@ -61,7 +67,7 @@ def parse_args():
                     help="context of one more decode point at the default batch (0: none)")
     ap.add_argument("--serve-seqs", type=int, default=256,
                     help="requests of the reference's benchmark workload through LLM.generate (0: not run)")
-    ap.add_argument("--design", default=None, choices=["nozurax", "mafarax"],
+    ap.add_argument("--design", default=None, choices=["nozurax", "mafarax", "kirisun"],
                     help="measure this design beside Qwen3 at equal layer sizes instead of the default workload")
     ap.add_argument("--design-sizes", default="1024,2048,4096", help="model widths of the --design measurement")
     return ap.parse_args()
@@ -83,11 +89,24 @@ def mafarax_config(width: int, layers: int, dtype: str) -> dict:
     return _mafarax(layers, width, heads, kv, dim, dim, inner, DESIGN_VOCAB, chunk=1024, dtype=dtype)
 
 
+def kirisun_config(width: int, layers: int, dtype: str) -> dict:
+    """A Kirisun model of the width's layer sizes: delta-rule layers with as many value heads of 128 channels as
+    the dense model has query heads (a state of 128 x 128 a head) and attention layers with the dense model's heads
+    (a window of 1024 positions that keeps the first 4, scores capped at 50, half the head rotated) in turn; 32
+    gated experts of an eighth of the dense inner size of which a token runs 8."""
+    from nano_vllm_amd.models.shapes import _kirisun
+    heads, kv, dim, inner = DESIGN_SIZES[width]
+    return _kirisun(layers, width, heads, kv, dim, dim, inner, DESIGN_VOCAB, window=1024, dtype=dtype)
+
+
 def design_configs(width: int, layers: int, dtype: str, design: str = "nozurax"):
     """config.json of a Nozurax model and of the Qwen3 model with the same layer sizes (and, for the Mafarax
     measurement, of the Mafarax model first)."""
     if design == "mafarax":
         return {"mafarax": mafarax_config(width, layers, dtype), **design_configs(width, layers, dtype)}
+    if design == "kirisun":
+        return {"kirisun": kirisun_config(width, layers, dtype), "mafarax": mafarax_config(width, layers, dtype),
+                "qwen3": design_configs(width, layers, dtype)["qwen3"]}
     heads, kv, dim, inner = DESIGN_SIZES[width]
     att = {"type": "attention", "mlp": {"kind": "dense", "ff": inner},
            "mixer": {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
@@ -176,7 +195,7 @@ def design_run(args):
             torch.cuda.empty_cache()
     first = out[next(iter(out))]
     line = {"metric": f"--design {args.design}: prefill tok/s @ {T} tokens and decode tok/s @ batch {B}, context {ctx}, "
-                      f"{layers} layers, beside {'Nozurax and ' if args.design == 'mafarax' else ''}Qwen3 at equal layer sizes",
+                      f"{layers} layers, beside {', '.join(n.capitalize() for n in first if n != args.design)} at equal layer sizes",
             "value": first[args.design]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": first[args.design]["decode_ms_per_step"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",

@@ -1,10 +1,12 @@
-from .model_config import (ChunkAttentionConfig, ConfigError, ExpertsConfig, MafaraxConfig, MafaraxLayer, NozuraxConfig,
-                           NozuraxLayer, Qwen3Config, StateSpaceConfig, canonical_dtype, read_config_json)
+from .model_config import (ChannelDeltaConfig, ChunkAttentionConfig, ConfigError, ExpertsConfig, GatedAttentionConfig,
+                           KirisunConfig, KirisunLayer, MafaraxConfig, MafaraxLayer, NozuraxConfig, NozuraxLayer, Qwen3Config,
+                           SoftmaxExpertsConfig, StateSpaceConfig, canonical_dtype, read_config_json)
 from .engine_config import EngineConfig
 from .registry import (Architecture, register_architecture, get_architecture,
                        architecture_of, known_architectures)
 
 __all__ = ["ConfigError", "Qwen3Config", "NozuraxConfig", "NozuraxLayer", "MafaraxConfig", "MafaraxLayer",
-           "ChunkAttentionConfig", "StateSpaceConfig", "ExpertsConfig", "canonical_dtype", "read_config_json", "EngineConfig",
+           "ChunkAttentionConfig", "StateSpaceConfig", "ExpertsConfig", "KirisunConfig", "KirisunLayer", "GatedAttentionConfig",
+           "ChannelDeltaConfig", "SoftmaxExpertsConfig", "canonical_dtype", "read_config_json", "EngineConfig",
            "Architecture", "register_architecture", "get_architecture", "architecture_of",
            "known_architectures"]

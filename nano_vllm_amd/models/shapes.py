@@ -1,7 +1,7 @@
 """Named config.json contents for runs with random weights (there is no checkpoint to read
 them from): two tiny test shapes and the Qwen3 dense sizes that the benchmarks use, three
-Nozurax shapes (a tiny one, and layers of the Qwen3 1.7B and 8B sizes) and two Mafarax shapes (a tiny
-one, and layers of the Qwen3 1.7B sizes).  These are
+Nozurax shapes (a tiny one, and layers of the Qwen3 1.7B and 8B sizes), two Mafarax shapes (a tiny
+one, and layers of the Qwen3 1.7B sizes) and two Kirisun shapes of the same kind.  These are
 inputs, as a model folder's config.json is; nothing in the model code reads them.
 
     python -m nano_vllm_amd.cli random-model --shape qwen3-8b --config-only --out DIR
@@ -57,7 +57,33 @@ def _mafarax(layers, width, heads, kv_heads, dim, vdim, inner, vocab, chunk, eps
             "layers": [layer] * layers, "torch_dtype": dtype}
 
 
+def _kirisun(layers, width, heads, kv_heads, dim, vdim, inner, vocab, window, keep_first=4, eps=1e-6, dtype="bfloat16",
+             rot=None, factor=2.0, softcap=50.0, delta_heads=None, delta_kv_heads=None, delta_dim=None, delta_vdim=None, conv=4,
+             rank=None, experts=32, top=8, residual_mult=0.5, pattern=("channel_delta", "attention")) -> dict:
+    """Layers that follow `pattern` in turn: the gated window attention (a cap on the scores, kept first positions,
+    half the head rotated) and the channel-wise delta rule (as many value heads of the same size as the attention's
+    query heads unless named), each with `top` of `experts` gated experts of inner / top each (a token runs the dense
+    layer's inner size)."""
+    dh, dd, dv = delta_heads or heads, delta_dim or dim, delta_vdim or vdim
+    mlp = {"kind": "moe", "expert": {"ff": max(1, inner // top)}, "router": {"experts": experts, "top": top}}
+    kinds = {
+        "attention": {"type": "attention", "mlp": mlp,
+                      "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5,
+                                "softcap": softcap, "mask": {"size": window, "keep_first": keep_first},
+                                "rot": {"dims": rot or dim // 2, "base": 1e6, "scaling": {"factor": factor}}}},
+        "channel_delta": {"type": "channel_delta", "mlp": mlp,
+                          "mixer": {"heads": dh, "kv_heads": delta_kv_heads or dh, "dim": dd, "vdim": dv, "conv": conv,
+                                    "decay_rank": rank or max(1, dd // 2), "gate_rank": rank or max(1, dd // 2)}},
+    }
+    return {"architecture": "Kirisun", "vocab": vocab, "width": width, "norm": {"eps": eps}, "residual_mult": residual_mult,
+            "embedding": {"scale": float(width) ** 0.5}, "layers": [kinds[pattern[i % len(pattern)]] for i in range(layers)],
+            "torch_dtype": dtype}
+
+
 SHAPES: Dict[str, dict] = {
+    "kirisun-tiny": _kirisun(4, 64, 4, 2, 16, 24, 96, 256, window=12, keep_first=3, eps=1e-5, dtype="float32", rot=8, softcap=5.0,
+                             delta_heads=4, delta_kv_heads=2, delta_dim=12, delta_vdim=8, conv=3, rank=3, experts=6, top=2),
+    "kirisun-1b": _kirisun(16, 2048, 16, 8, 128, 128, 6144, 32768, window=1024),
     "mafarax-tiny": _mafarax(3, 64, 4, 2, 16, 24, 96, 256, chunk=12, eps=1e-5, dtype="float32", rot=8, ssm_heads=4,
                              ssm_vdim=8, state=12, groups=2, conv=3, norm_groups=2, experts=6, top=2, group_count=3,
                              group_keep=2, logit_scale=1.5),

@@ -85,16 +85,14 @@ def sink_softmax(scores):
     return e / (math.exp(-m) + e.sum())
 
 
-def gated_attention(h, m, w, p, eps):
-    T = h.shape[0]
-    H, G, D, DV = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = unit_mean((h @ w[p + ".q"].T).reshape(T, H, D), eps) * w[p + ".q.norm"]
-    k = unit_mean((h @ w[p + ".k"].T).reshape(T, G, D), eps) * w[p + ".k.norm"]
-    q, k = turn_heads(q, m.get("rot")), turn_heads(k, m.get("rot"))
-    v = (h @ w[p + ".v"].T).reshape(T, G, DV)
+def attend(q, k, v, m, rows=None):
+    """q [T, H, D], k [T, G, D], v [T, G, DV] of a whole sequence, ready (normed, turned): every head's output
+    [T, H, DV] (rows: only these positions are computed, the others stay zero)."""
+    T, H = q.shape[0], q.shape[1]
+    G, DV = k.shape[1], v.shape[2]
     cap = m.get("softcap")
-    heads_out = torch.zeros(T, H, DV, dtype=h.dtype)
-    for i in range(T):
+    heads_out = torch.zeros(T, H, DV, dtype=q.dtype)
+    for i in (range(T) if rows is None else rows):
         js = [j for j in range(i + 1) if sees(i, j, m.get("mask"))]
         for a in range(H):
             g = a // (H // G)
@@ -102,8 +100,18 @@ def gated_attention(h, m, w, p, eps):
             if cap:
                 s = cap * torch.tanh(s / cap)
             heads_out[i, a] = sink_softmax(s) @ v[js, g]
+    return heads_out
+
+
+def gated_attention(h, m, w, p, eps):
+    T = h.shape[0]
+    H, G, D, DV = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    q = unit_mean((h @ w[p + ".q"].T).reshape(T, H, D), eps) * w[p + ".q.norm"]
+    k = unit_mean((h @ w[p + ".k"].T).reshape(T, G, D), eps) * w[p + ".k.norm"]
+    q, k = turn_heads(q, m.get("rot")), turn_heads(k, m.get("rot"))
+    v = (h @ w[p + ".v"].T).reshape(T, G, DV)
     gate = torch.sigmoid(h @ w[p + ".g"].T)
-    return (heads_out.reshape(T, H * DV) * gate) @ w[p + ".o"].T
+    return (attend(q, k, v, m).reshape(T, H * DV) * gate) @ w[p + ".o"].T
 
 
 def short_conv(u, kernel):
@@ -123,29 +131,36 @@ def unit_sum(x):
     return x / torch.sqrt(x.pow(2).sum(dim=-1, keepdim=True) + 1e-6)
 
 
-def channel_delta(h, m, w, p, eps):
-    T = h.shape[0]
+def delta_of_projections(q_in, k_in, v_in, b_in, a_in, g_in, m, w, p, eps):
+    """The mixer between its input projections and its output projection: q_in, k_in [T, G D], v_in [T, H DV],
+    b_in [T, H], a_in [T, H D] (before dt_bias), g_in [T, H DV] (before the sigmoid)."""
+    T = q_in.shape[0]
     H, G, D, DV = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = silu(short_conv(h @ w[p + ".q"].T, w[p + ".q.conv"])).reshape(T, G, D)
-    k = silu(short_conv(h @ w[p + ".k"].T, w[p + ".k.conv"])).reshape(T, G, D)
-    v = silu(short_conv(h @ w[p + ".v"].T, w[p + ".v.conv"])).reshape(T, H, DV)
+    q = silu(short_conv(q_in, w[p + ".q.conv"])).reshape(T, G, D)
+    k = silu(short_conv(k_in, w[p + ".k.conv"])).reshape(T, G, D)
+    v = silu(short_conv(v_in, w[p + ".v.conv"])).reshape(T, H, DV)
     q = unit_sum(q) * D ** -0.5
     k = unit_sum(k)
-    beta = torch.sigmoid(h @ w[p + ".b"].T)                                             # [T, H]
-    step = torch.log1p(torch.exp((h @ w[p + ".a1"].T) @ w[p + ".a2"].T + w[p + ".dt_bias"])).reshape(T, H, D)
+    beta = torch.sigmoid(b_in)                                                          # [T, H]
+    step = torch.log1p(torch.exp(a_in + w[p + ".dt_bias"])).reshape(T, H, D)
     decay = torch.exp(-torch.exp(w[p + ".A_log"])[None, :, None] * step)                # [T, H, D]
-    o = torch.zeros(T, H, DV, dtype=h.dtype)
+    o = torch.zeros(T, H, DV, dtype=q_in.dtype)
     for a in range(H):
         g = a // (H // G)
-        S = torch.zeros(D, DV, dtype=h.dtype)
+        S = torch.zeros(D, DV, dtype=q_in.dtype)
         for t in range(T):
             S = decay[t, a][:, None] * S
             u = beta[t, a] * (v[t, a] - S.T @ k[t, g])
             S = S + torch.outer(k[t, g], u)
             o[t, a] = S.T @ q[t, g]
     o = unit_mean(o, eps) * w[p + ".norm"]
-    gate = torch.sigmoid((h @ w[p + ".g1"].T) @ w[p + ".g2"].T)
-    return (o.reshape(T, H * DV) * gate) @ w[p + ".o"].T
+    return o.reshape(T, H * DV) * torch.sigmoid(g_in)
+
+
+def channel_delta(h, m, w, p, eps):
+    y = delta_of_projections(h @ w[p + ".q"].T, h @ w[p + ".k"].T, h @ w[p + ".v"].T, h @ w[p + ".b"].T,
+                             (h @ w[p + ".a1"].T) @ w[p + ".a2"].T, (h @ w[p + ".g1"].T) @ w[p + ".g2"].T, m, w, p, eps)
+    return y @ w[p + ".o"].T
 
 
 def chosen_experts(z, top):

@@ -1,0 +1,790 @@
+"""Kirisun: every mechanism alone, and the model through the step function and the engine, against
+the plain implementation (tests/plain_kirisun.py).  Each test runs on the CPU stand-ins of the
+device operations (tests/torch_kernels.py; this checks the stand-ins and the host logic) and, marked
+gpu, on the HIP kernels."""
+import json
+import math
+import random
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+import helpers as H
+import kirisun_cases as K
+import plain_kirisun as plain
+from nano_vllm_amd import LLM, SamplingParams
+from nano_vllm_amd.config import ConfigError, KirisunConfig, architecture_of
+from nano_vllm_amd.parts.base import NormedAddend
+from torch_kernels import TorchKernels, new_caches
+
+BACKENDS = ["cpu", pytest.param("hip", marks=pytest.mark.gpu)]
+DTYPES = [torch.float32, torch.bfloat16]
+_hip = {}
+
+
+def _kernels(backend, dtype=torch.float32):
+    if backend == "cpu":
+        return TorchKernels("cpu", dtype), "cpu"
+    from nano_vllm_amd.kernels import HipKernels
+    if dtype not in _hip:
+        _hip[dtype] = HipKernels("cuda:0", dtype, quiet=True)
+    return _hip[dtype], "cuda:0"
+
+
+def _tol(dtype):
+    return 3e-5 if dtype == torch.float32 else 2e-2
+
+
+def _close(got, want, dtype, what="", tol=None):
+    e = float((got.double().cpu() - want.double()).abs().max() / max(float(want.double().abs().max()), 1e-9))
+    assert e < (tol or _tol(dtype)), f"{what}: differs by {e:.2e} of the largest"
+
+
+# ------------------------------------------------------------------------------ configuration
+def test_config_is_read_written_and_refused():
+    for name, c in K.CONFIGS.items():
+        d = c["cfg"].to_dict()
+        arch = architecture_of(d)
+        assert arch.name == "Kirisun"
+        again = arch.parse_config(json.loads(json.dumps(d)))
+        assert again == c["cfg"].__class__(**{**c["cfg"].__dict__, "dtype": again.dtype}), name
+    d = K.CONFIGS["a"]["cfg"].to_dict()
+    # what may be left out: the cap, the mask, the kept positions, the rotation and its scaling, the feed-forward,
+    # the residual multiplier and the embedding's scale
+    e = json.loads(json.dumps(d))
+    att = e["layers"][1]["mixer"]
+    del att["softcap"], att["mask"]["keep_first"], att["rot"]["scaling"]
+    del e["residual_mult"], e["embedding"]
+    e["layers"][2]["mixer"].pop("mask"), e["layers"][2]["mixer"].pop("rot")
+    e["layers"][2]["mixer"]["softcap"] = None
+    cfg = KirisunConfig.from_dict(e)
+    m1, m2 = cfg.layers[1].mixer, cfg.layers[2].mixer
+    assert (m1.softcap, m1.window, m1.keep_first, m1.rot_factor) == (None, 10, 0, 1.0)
+    assert (m2.window, m2.keep_first, m2.rot_dims, m2.softcap) == (None, 0, 0, None)
+    assert cfg.residual_mult == 1.0 and cfg.embedding_scale == 1.0 and cfg.layers[1].mlp is None
+
+    def broken(change):
+        e = json.loads(json.dumps(d))
+        change(e)
+        with pytest.raises(ConfigError):
+            KirisunConfig.from_dict(e)
+    broken(lambda e: e["layers"][0].update(type="other"))
+    broken(lambda e: e["layers"][1]["mixer"].update(kv_heads=3))
+    broken(lambda e: e["layers"][1]["mixer"]["rot"].update(dims=7))
+    broken(lambda e: e["layers"][1]["mixer"]["rot"].update(dims=18))
+    broken(lambda e: e["layers"][1]["mixer"].pop("scale"))
+    broken(lambda e: e["layers"][0]["mixer"].pop("conv"))
+    broken(lambda e: e["layers"][0]["mlp"]["router"].update(top=7))
+    broken(lambda e: e["norm"].update(eps=0.0))
+    broken(lambda e: e.update(layers=[]))
+
+
+def test_the_checkpoint_is_read_by_its_own_names():
+    from safetensors import safe_open
+    folder = K.model_folder("a")
+    with safe_open(folder + "/model.safetensors", "pt") as f:
+        names = set(f.keys())
+    for n in ("embed", "head", "final.norm", "l0.norm1", "l0.norm1b", "l0.norm2", "l0.norm2b", "l0.mix.q", "l0.mix.q.conv",
+              "l0.mix.k.conv", "l0.mix.v.conv", "l0.mix.b", "l0.mix.a1", "l0.mix.a2", "l0.mix.g1", "l0.mix.g2", "l0.mix.dt_bias",
+              "l0.mix.A_log", "l0.mix.norm", "l0.mix.o", "l0.mlp.router", "l0.mlp.router.b", "l0.mlp.e5.gate", "l0.mlp.e0.up",
+              "l0.mlp.e3.down", "l1.mix.q.norm", "l1.mix.k.norm", "l1.mix.g", "l1.mix.v", "l1.mix.o"):
+        assert n in names, n
+    assert not any(n.startswith("l1.mlp") or n.startswith("l1.norm2") for n in names)
+    with safe_open(folder + "/model.safetensors", "pt") as f:
+        assert tuple(f.get_tensor("l0.mix.a1").shape) == (5, 48) and tuple(f.get_tensor("l0.mix.g2").shape) == (32, 3)
+        assert tuple(f.get_tensor("l0.mix.a2").shape) == (48, 5) and tuple(f.get_tensor("l0.mix.q.conv").shape) == (24, 3)
+
+
+# ------------------------------------------------------------------------------ the stream
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_scaled_embedding_starts_a_float_stream(backend, dtype):
+    k, dev = _kernels(backend, dtype)
+    g = torch.Generator().manual_seed(1)
+    table = torch.randn((50, 36), generator=g).to(dtype)
+    ids = torch.tensor([3, 49, 0, 3, 17], dtype=torch.int32)
+    got = k.embedding_scaled(table.to(dev), ids.to(dev), 13.37)
+    assert got.dtype == torch.float32
+    want = table[ids.long()].double() * 13.37
+    assert float((got.cpu().double() - want).abs().max()) < 1e-5 * float(want.abs().max())     # no rounding to the element type
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width,mult", [(48, 0.5), (20, 1.0), (320, 0.3), (1000, 2.0)])
+def test_a_normed_addend_goes_into_the_float_stream(backend, dtype, width, mult):
+    """r <- r + mult * n_a(a), y = n(r): the stream stays float32 (far beyond bfloat16's grain), y is rounded once."""
+    k, dev = _kernels(backend, dtype)
+    g = torch.Generator().manual_seed(width)
+    rows = 9
+    a = (torch.randn((rows, width), generator=g) * 3).to(dtype)
+    r = torch.randn((rows, width), generator=g) * 40 + 1000.0
+    wa, w = 1 + 0.3 * torch.randn(width, generator=g), 1 + 0.3 * torch.randn(width, generator=g)
+    if dtype == torch.bfloat16:
+        wa, w = wa.to(dtype), w.to(dtype)
+    stream = r.clone().to(dev)
+    y, res = k.stream_rms_norm((NormedAddend(a.to(dev), wa.to(dev), 1e-5, mult),), stream, w.to(dev), 1e-6)
+    want_r = r.double() + mult * plain.unit_mean(a.double(), 1e-5) * wa.double()
+    want_y = plain.unit_mean(want_r, 1e-6) * w.double()
+    assert res.dtype == torch.float32 and res.data_ptr() == stream.data_ptr()
+    assert float((res.cpu().double() - want_r).abs().max()) < 2e-4                         # the stream itself: float32 of ~1000
+    _close(y, want_y, dtype, "normed stream")
+    # two in a row and the stream alone (the model's last norm after a layer without feed-forward)
+    y2, res = k.stream_rms_norm((NormedAddend(a.to(dev), w.to(dev), 1e-6, 1.0),), res, wa.to(dev), 1e-5)
+    want_r2 = want_r + plain.unit_mean(a.double(), 1e-6) * w.double()
+    _close(y2, plain.unit_mean(want_r2, 1e-5) * wa.double(), dtype, "second")
+
+
+# ------------------------------------------------------------------------------ query and key preparation
+def _turn_at(x, rot, p):
+    """x [heads, dim] at position p, by the plain rotation (which turns row t by first_position + t)."""
+    return plain.turn_heads(x[None], rot, first_position=p)[0]
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq,hkv,D,DV,R,page,factor", [(4, 2, 16, 24, 8, 8, 4.0), (2, 2, 24, 8, 24, 4, 1.0), (3, 1, 10, 10, 0, 16, 1.0),
+                                                        (8, 2, 64, 64, 32, 32, 2.0), (2, 1, 128, 96, 64, 16, 8.0)])
+def test_head_norms_then_rotation_of_a_part_of_the_head_and_store(backend, dtype, hq, hkv, D, DV, R, page, factor):
+    k, dev = _kernels(backend, dtype)
+    g = torch.Generator().manual_seed(3)
+    positions = [0, 1, 2, 5, 63, 64, 1000, 4097, 30000]
+    T = len(positions)
+    width = hq * D + hkv * D + hkv * DV
+    qkv = (torch.randn((T, width), generator=g) * 2.5).to(dtype)
+    qw, kw = 1 + 0.4 * torch.randn(D, generator=g), 1 + 0.4 * torch.randn(D, generator=g)
+    if dtype == torch.bfloat16:
+        qw, kw = qw.to(dtype), kw.to(dtype)
+    base, eps = 500.0, 1e-5
+    pos = torch.tensor(positions, dtype=torch.int32, device=dev)
+    extra = {}
+    if R:
+        inv_freq = (1.0 / (base ** (torch.arange(0, R, 2, dtype=torch.float) / R)) / factor).to(dev)
+        extra["rot_table"] = k.rotary_step_table(inv_freq, pos)
+    kc, vc = new_caches(3, hkv, D, page, dtype, dev, v_head_dim=DV)
+    slots = torch.tensor([5, 0, 2 * page + 1, -1, page, 3, 1, 2, 2 * page + 2][:T], dtype=torch.int32, device=dev)
+    q = k.qk_rownorm_store(qkv.clone().to(dev), hq, hkv, D, DV, qw.to(dev), kw.to(dev), eps, pos, 0.0, 1, slots, kc, vc,
+                           norm_per_head=True, **extra)
+    rot = {"dims": R, "base": base, "scaling": {"factor": factor}} if R else None
+
+    def prepared(x, heads, w):
+        x = plain.unit_mean(x.double().reshape(T, heads, D), eps) * w.double()
+        return torch.stack([_turn_at(x[i], rot, p) for i, p in enumerate(positions)])
+    tol = 2e-2 if dtype == torch.bfloat16 else 2e-3       # float angles of large positions
+    _close(q.reshape(T, hq, D), prepared(qkv[:, : hq * D], hq, qw), dtype, "q", tol)
+    want_k = prepared(qkv[:, hq * D: hq * D + hkv * D], hkv, kw)
+    vt = vc.shape[4]
+    for i, s in enumerate(slots.tolist()):
+        if s < 0:
+            continue
+        _close(kc[s // page, :, s % page, :], want_k[i], dtype, f"k {i}", tol)
+        assert torch.equal(vc[s // page, :, (s % page) // vt, :, (s % page) % vt].cpu().float(),
+                           qkv[i, hq * D + hkv * D:].reshape(hkv, DV).float()), i
+
+
+def test_the_plain_rotation_turns_row_t_by_position_t():
+    rot = {"dims": 6, "base": 50.0, "scaling": {"factor": 1.5}}
+    x = torch.randn(4, 2, 8, dtype=torch.float64)
+    got = plain.turn_heads(x, rot)
+    for t in range(4):
+        for i in range(3):
+            a = t * 50.0 ** (-2.0 * i / 6) / 1.5
+            assert abs(float(got[t, 1, i]) - (float(x[t, 1, i]) * math.cos(a) - float(x[t, 1, i + 3]) * math.sin(a))) < 1e-12
+            assert abs(float(got[t, 1, i + 3]) - (float(x[t, 1, i + 3]) * math.cos(a) + float(x[t, 1, i]) * math.sin(a))) < 1e-12
+    assert torch.equal(got[..., 6:], x[..., 6:])
+
+
+# ------------------------------------------------------------------------------ attention
+def _attention_case(dtype, dev, hq, hkv, D, DV, page, lens, q_lens, seed, window, keep, boost=None, free_passed=False):
+    """Requests with kv lengths `lens`, the last q_lens of which are this step's queries; keys and values over
+    shuffled pages (what unused slots hold must not matter: NaN).  boost = (request, key): that key is made the
+    one its request's queries prefer by far.  free_passed: pages wholly before the window of a request's first
+    query, the pages of the kept first positions aside, are taken out of its table, as the cache manager gives
+    them back."""
+    rng = random.Random(seed)
+    g = torch.Generator().manual_seed(seed)
+    S = len(lens)
+    pages_per = [(n + page - 1) // page for n in lens]
+    total = sum(pages_per) + 2
+    order = list(range(total))
+    rng.shuffle(order)
+    kc, vc = new_caches(total, hkv, D, page, dtype, dev, v_head_dim=DV)
+    kc.fill_(float("nan")), vc.fill_(float("nan"))
+    vt = vc.shape[4]
+    tables = torch.full((S, max(pages_per)), -1, dtype=torch.int32)
+    ks, vs, qs, token_seq, positions = [], [], [], [], []
+    for s, n in enumerate(lens):
+        mine = [order.pop() for _ in range(pages_per[s])]
+        held = set(range(len(mine)))
+        if free_passed and window is not None:
+            first_needed = max(0, (n - q_lens[s]) - window + 1) // page
+            held = set(range(first_needed, len(mine))) | set(range((keep + page - 1) // page))
+        for p in held:
+            tables[s, p] = mine[p]
+        kk = torch.randn((n, hkv, D), generator=g).to(dtype)
+        vv = torch.randn((n, hkv, DV), generator=g).to(dtype)
+        qq = torch.randn((n, hq, D), generator=g).to(dtype)
+        if boost is not None and boost[0] == s:
+            kk[boost[1]] = 0
+            kk[boost[1], :, 0] = 8.0
+            qq[:] = 0
+            qq[:, :, 0] = 8.0
+        for j in range(n):
+            if j // page in held:
+                kc[mine[j // page], :, j % page, :] = kk[j].to(dev)
+                vc[mine[j // page], :, (j % page) // vt, :, (j % page) % vt] = vv[j].to(dev)
+        ks.append(kk), vs.append(vv), qs.append(qq)
+        token_seq += [s] * q_lens[s]
+        positions += list(range(n - q_lens[s], n))
+    q = torch.cat([qs[s][lens[s] - q_lens[s]:] for s in range(S)]).reshape(sum(q_lens), hq * D).contiguous().to(dev)
+    assert all(a == 1 or b != 1 for a, b in zip(q_lens, q_lens[1:])), "single tokens come first in a batch"
+    batch = SimpleNamespace(
+        num_seqs=S, num_tokens=sum(q_lens), token_seq=torch.tensor(token_seq, dtype=torch.int32, device=dev),
+        positions=torch.tensor(positions, dtype=torch.int32, device=dev), max_kv_len=max(lens), max_q_len=max(q_lens),
+        kv_lens=torch.tensor(lens, dtype=torch.int32, device=dev),
+        cu_seqlens_q=torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32, device=dev),
+        num_decode=next((i for i, n in enumerate(q_lens) if n != 1), len(q_lens)), q_lens=list(q_lens),
+        starts=[n - m for n, m in zip(lens, q_lens)],
+        groups=[SimpleNamespace(block_tables=tables.to(dev), slot_mapping=None)])
+    return q, kc, vc, batch, (qs, ks, vs)
+
+
+def _plain_attention(qs, ks, vs, lens, q_lens, scale, cap, window, keep):
+    m = {"scale": scale, "softcap": cap, "mask": None if window is None else {"size": window, "keep_first": keep}}
+    rows = []
+    for q, k, v, n, c in zip(qs, ks, vs, lens, q_lens):
+        o = plain.attend(q.double(), k.double(), v.double(), m, rows=range(n - c, n))
+        rows.append(o[n - c:].reshape(c, -1))
+    return torch.cat(rows)
+
+
+def _attend(k, dev, q, hq, hkv, D, DV, kc, vc, batch, scale, cap, window, keep):
+    sinks = torch.zeros(hq, dtype=torch.float32, device=dev)
+    got = k.paged_attention(q, hq, hkv, D, kc, vc, batch, 0, scale, window, v_head_dim=DV, sinks=sinks, softcap=cap,
+                            keep_first=keep)
+    k.check_faults()
+    return got
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq,hkv,D,DV,page,window,keep,cap,lens,q_lens", [
+    (4, 2, 16, 24, 8, 10, 3, 4.0, [31, 10, 11, 57, 40], [1, 1, 1, 57, 13]),     # decoded tokens whose window just left, holds and passed the kept ones
+    (6, 2, 24, 40, 16, 33, 19, 6.0, [200, 67, 150], [1, 67, 85]),                # kept positions over more than a page
+    (3, 3, 6, 10, 4, 1, 2, 2.0, [9, 5], [1, 5]),                                 # a window of one position
+    (2, 1, 64, 64, 32, 48, 4, 30.0, [97, 150], [1, 85]),                         # sizes of the matrix-core kind
+    (2, 2, 8, 8, 4, 4096, 5, None, [70, 130], [1, 130]),                         # a window longer than every request, no cap
+    (2, 1, 10, 10, 4, None, 0, 1.5, [50, 21], [1, 21]),                          # no window at all
+    (4, 1, 64, 64, 16, 40, 0, 50.0, [120, 90], [1, 60]),                         # a window without kept positions
+    (8, 2, 128, 128, 64, 96, 70, 20.0, [500, 260], [1, 260])])
+def test_capped_window_attention_with_kept_first_positions_and_a_sink(backend, dtype, hq, hkv, D, DV, page, window, keep, cap,
+                                                                      lens, q_lens):
+    if backend == "cpu" and D == 128:
+        pytest.skip("minutes on the stand-in's loops")
+    k, dev = _kernels(backend, dtype)
+    for free_passed in (False, True):
+        q, kc, vc, batch, (qs, ks, vs) = _attention_case(dtype, dev, hq, hkv, D, DV, page, lens, q_lens, 5, window, keep,
+                                                         free_passed=free_passed)
+        got = _attend(k, dev, q, hq, hkv, D, DV, kc, vc, batch, 0.3, cap, window, keep)
+        _close(got, _plain_attention(qs, ks, vs, lens, q_lens, 0.3, cap, window, keep), dtype, (window, keep, free_passed))
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_the_cap_and_the_sink_show(backend):
+    """Scores far beyond the cap: without it the softmax would be one-hot, with it the largest score is the cap.  A
+    lone key of score s gets e^s / (1 + e^s) of the weight, not all of it."""
+    k, dev = _kernels(backend)
+    D, DV, page = 8, 4, 4
+    q, kc, vc, batch, (qs, ks, vs) = _attention_case(torch.float32, dev, 1, 1, D, DV, page, [1], [1], 2, None, 0)
+    s = float(qs[0][0, 0] @ ks[0][0, 0]) * 0.25
+    got = _attend(k, dev, q, 1, 1, D, DV, kc, vc, batch, 0.25, None, None, 0)
+    assert float((got.cpu()[0] - vs[0][0, 0] * (math.exp(s) / (1 + math.exp(s)))).abs().max()) < 1e-5
+    q, kc, vc, batch, (qs, ks, vs) = _attention_case(torch.float32, dev, 1, 1, D, DV, page, [6], [1], 3, None, 0, boost=(0, 2))
+    got = _attend(k, dev, q, 1, 1, D, DV, kc, vc, batch, 1.0, 1.0, None, 0).cpu()[0]
+    # the preferred key's score of 64 is capped to 1, so the others keep a share: uncapped it would take everything
+    e = torch.exp(torch.tanh(8.0 * ks[0][:, 0, 0].double()))
+    assert abs(float(e[2]) - math.e) < 1e-9
+    want = (e / (1 + e.sum())) @ vs[0][:, 0].double()
+    assert float((got.double() - want).abs().max()) < 1e-5 and float((got - vs[0][2, 0]).abs().max()) > 0.1
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("D,DV", [(16, 24), (64, 64)])
+def test_a_key_just_inside_and_just_outside_the_window_and_the_kept_positions(backend, dtype, D, DV):
+    """One key that every query prefers by far: at the window's oldest place and one before it, at the last kept
+    position and the one after it, hundreds of positions back among the kept; in a prompt's portion and by a
+    decoded token, on tables whose passed pages went back."""
+    k, dev = _kernels(backend, dtype)
+    window, keep, page = 40, 6, 16
+    for q_len in (1, 25):
+        for n in (300, 337, 47, 41, 40):
+            last = n - 1
+            cases = [(last, True), (last - window + 1, True), (last - window, last - window < keep), (keep - 1, True),
+                     (keep, last - keep < window), (0, True), (last - window - 100, False)]
+            for key, seen in cases:
+                if key < 0 or key > last:
+                    continue
+                q, kc, vc, batch, (qs, ks, vs) = _attention_case(dtype, dev, 2, 1, D, DV, page, [n], [q_len], 7, window, keep,
+                                                                 boost=(0, key), free_passed=True)
+                got = _attend(k, dev, q, 2, 1, D, DV, kc, vc, batch, 1.0, 80.0, window, keep)
+                row = got[-1].float().cpu().reshape(2, DV)
+                hit = float((row[0] - vs[0][key, 0].float()).abs().max()) < 0.05
+                assert hit == seen, (q_len, n, key, seen)
+                _close(got, _plain_attention(qs, ks, vs, [n], [q_len], 1.0, 80.0, window, keep), dtype, (q_len, n, key))
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_sigmoid_gate(backend, dtype):
+    k, dev = _kernels(backend, dtype)
+    g = torch.Generator().manual_seed(8)
+    both = (torch.randn((7, 200), generator=g) * 3).to(dtype).to(dev)
+    x, gate = both[:, :100], both[:, 100:]                                    # rows wider than what is read
+    want = x.double().cpu() * torch.sigmoid(gate.double().cpu())
+    _close(k.sigmoid_mul(x.clone(), gate), want, dtype, "gate")
+
+
+# ------------------------------------------------------------------------------ experts
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("experts,top", [(6, 2), (4, 1), (5, 3), (3, 3), (12, 3), (64, 6), (15, 2)])
+def test_the_largest_logits_are_chosen_and_weighted_among_themselves(backend, experts, top):
+    k, dev = _kernels(backend)
+    g = torch.Generator().manual_seed(experts * 10 + top)
+    logits = torch.randn((40, experts), generator=g) * 2
+    bias = torch.randn(experts, generator=g)
+    logits[3] = -bias                                    # all equal after the bias: whichever are chosen weigh the same
+    logits[4, experts - 1] += 50.0                       # one far ahead: it takes nearly all the weight
+    ids, weights = k.moe_route(logits.to(dev), top, 1, 1, 1.0, routing="softmax_top", bias=bias.to(dev))
+    ids, weights = ids.cpu(), weights.cpu()
+    for t in range(logits.shape[0]):
+        if t == 3:
+            continue
+        want_ids, want_w = plain.chosen_experts(logits[t].double() + bias.double(), top)
+        order = sorted(range(top), key=lambda c: (-float(weights[t, c]), int(ids[t, c])))
+        assert [int(ids[t, c]) for c in order] == want_ids, t
+        assert float((weights[t][order].double() - want_w).abs().max()) < 1e-5
+        assert abs(float(weights[t].sum()) - 1.0) < 1e-5
+    assert len(set(ids[3].tolist())) == top and float((weights[3] - 1.0 / top).abs().max()) < 1e-6
+    assert int(ids[4][weights[4].argmax()]) == experts - 1 and (top == 1 or float(weights[4].max()) > 0.999)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tokens,width,ff,experts,top", [(1, 48, 20, 6, 2), (7, 20, 9, 5, 3), (150, 72, 30, 10, 2), (33, 128, 64, 8, 3),
+                                                          (300, 64, 32, 3, 1), (5, 256, 72, 10, 3)])
+def test_the_gated_experts_products(backend, dtype, tokens, width, ff, experts, top):
+    k, dev = _kernels(backend, dtype)
+    g = torch.Generator().manual_seed(tokens)
+    x = torch.randn((tokens, width), generator=g).to(dtype)
+    w = {}
+    for e in range(experts):
+        w[f".e{e}.gate"] = (torch.randn((ff, width), generator=g) * width ** -0.5).to(dtype)
+        w[f".e{e}.up"] = (torch.randn((ff, width), generator=g) * width ** -0.5).to(dtype)
+        w[f".e{e}.down"] = (torch.randn((width, ff), generator=g) * ff ** -0.5).to(dtype)
+    ids = torch.stack([torch.randperm(experts, generator=g)[:top] for _ in range(tokens)]).to(torch.int32)
+    if tokens > 100:
+        ids[:, 0] = 1                                      # one expert with more rows than a tile
+        ids[:, 1:] = torch.where(ids[:, 1:] == 1, torch.zeros_like(ids[:, 1:]) + (2 if experts > 2 else 0), ids[:, 1:])
+        if top > 2:
+            ids[:, 2] = 0
+    weights = torch.softmax(torch.randn((tokens, top), generator=g), -1)
+    up = torch.cat([torch.cat((w[f".e{e}.gate"], w[f".e{e}.up"])) for e in range(experts)]).contiguous()
+    down = torch.cat([w[f".e{e}.down"] for e in range(experts)]).contiguous()
+    got = k.moe_experts(x.to(dev), ids.to(dev), weights.to(dev), up.to(dev), down.to(dev), experts, act="silu", gated=True)
+    wd = {n: t.double() for n, t in w.items()}
+    want = torch.zeros((tokens, width), dtype=torch.float64)
+    for t in range(tokens):
+        for c in range(top):
+            want[t] += float(weights[t, c]) * plain.expert(x[t].double(), wd, f".e{int(ids[t, c])}")
+    _close(got, want, dtype, "experts", 3e-2 if dtype == torch.bfloat16 else None)
+
+
+# ------------------------------------------------------------------------------ the delta rule
+DELTA_SHAPES = [(4, 2, 12, 8, 3), (2, 2, 10, 14, 1), (3, 1, 5, 7, 5), (2, 1, 40, 70, 2), (4, 4, 64, 64, 4), (2, 1, 128, 128, 4),
+                (1, 1, 130, 20, 2)]          # heads, kv_heads, dim, vdim, taps
+
+
+def _delta_weights(shape, seed, dtype, slow=None):
+    heads, kv_heads, dim, vdim, taps = shape
+    g = torch.Generator().manual_seed(seed)
+    C = 2 * kv_heads * dim + heads * vdim
+    w = {"conv": (torch.randn((C, taps), generator=g) * 0.6).to(dtype), "dt_bias": torch.randn(heads * dim, generator=g) - 0.5,
+         "A_log": torch.log(0.05 + 1.5 * torch.rand(heads, generator=g)), "norm": 1 + 0.4 * torch.randn(vdim, generator=g)}
+    if slow is not None:
+        w["A_log"][slow] = -14.0           # a head that forgets next to nothing
+    return w
+
+
+def _delta_inputs(shape, T, seed, dtype):
+    heads, kv_heads, dim, vdim, taps = shape
+    g = torch.Generator().manual_seed(seed)
+    C = 2 * kv_heads * dim + heads * vdim
+    proj = (torch.randn((T, C + heads), generator=g) * 1.5).to(dtype)
+    decay_in = torch.randn((T, heads * dim), generator=g) * 1.5
+    gate_in = (torch.randn((T, heads * vdim), generator=g) * 2).to(dtype)
+    return proj, decay_in, gate_in
+
+
+def _plain_delta(shape, w, inputs, eps):
+    heads, kv_heads, dim, vdim, taps = shape
+    proj, decay_in, gate_in = (t.double() for t in inputs)
+    qk, vv = kv_heads * dim, heads * vdim
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim}
+    conv = w["conv"].double()
+    weights = {".q.conv": conv[:qk], ".k.conv": conv[qk:2 * qk], ".v.conv": conv[2 * qk:], ".dt_bias": w["dt_bias"].double(),
+               ".A_log": w["A_log"].double(), ".norm": w["norm"].double()}
+    return plain.delta_of_projections(proj[:, :qk], proj[:, qk:2 * qk], proj[:, 2 * qk:2 * qk + vv], proj[:, 2 * qk + vv:],
+                                      decay_in, gate_in, m, weights, "", eps)
+
+
+def _state_batch(dev, q_lens, starts, slots):
+    token_seq = [s for s, n in enumerate(q_lens) for _ in range(n)]
+    return SimpleNamespace(
+        num_seqs=len(q_lens), q_lens=list(q_lens), starts=list(starts),
+        num_decode=next((i for i, n in enumerate(q_lens) if n != 1), len(q_lens)),
+        token_seq=torch.tensor(token_seq, dtype=torch.int32, device=dev),
+        positions=torch.tensor([p for s, n in zip(starts, q_lens) for p in range(s, s + n)], dtype=torch.int32, device=dev),
+        cu_seqlens_q=torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32, device=dev),
+        seq_starts=torch.tensor(starts, dtype=torch.int32, device=dev),
+        state_slots=torch.tensor(slots, dtype=torch.int32, device=dev))
+
+
+def _new_states(dev, slots, shape, fill=float("nan")):
+    heads, kv_heads, dim, vdim, taps = shape
+    C = 2 * kv_heads * dim + heads * vdim
+    return (torch.full((slots, C, taps - 1), fill, dtype=torch.float32, device=dev),
+            torch.full((slots, heads, dim, vdim), fill, dtype=torch.float32, device=dev))
+
+
+def _run_delta(k, dev, shape, w, inputs, eps, states, q_lens, starts, slots):
+    heads, kv_heads, dim, vdim, taps = shape
+    proj, decay_in, gate_in = inputs
+    out = k.channel_delta(proj.to(dev), decay_in.to(dev).contiguous(), gate_in.to(dev), heads, kv_heads, dim, vdim, taps,
+                          w["conv"].to(dev), w["dt_bias"].to(dev), w["A_log"].to(dev), w["norm"].to(dev), eps, states[0], states[1],
+                          _state_batch(dev, q_lens, starts, slots))
+    k.check_faults()
+    return out
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", DELTA_SHAPES)
+def test_the_delta_rule_in_portions_of_every_size_and_token_by_token(backend, dtype, shape):
+    """One request of 45 tokens: whole, token by token, and in portions down to two tokens and shorter than the
+    convolution, on a slot that held NaN (a request's start reads nothing of what its slot held)."""
+    k, dev = _kernels(backend, dtype)
+    T, eps = 45, 1e-5
+    w = _delta_weights(shape, 11, dtype)
+    inputs = _delta_inputs(shape, T, 12, dtype)
+    want = _plain_delta(shape, w, inputs, eps)
+    cuttings = ([T], [1] * T, [2, 2, 1, 3, 1, 1, 2, 17, 5, 2, 9], [1, 44], [44, 1], [13, 2, 30])
+    for portions in cuttings[:3] if backend == "cpu" and shape[2] >= 64 else cuttings:
+        states = _new_states(dev, 3, shape)
+        outs, pos = [], 0
+        for n in portions:
+            part = tuple(t[pos:pos + n] for t in inputs)
+            outs.append(_run_delta(k, dev, shape, w, part, eps, states, [n], [pos], [1]))
+            pos += n
+        _close(torch.cat(outs), want, dtype, portions[:4], 4e-2 if dtype == torch.bfloat16 else 1e-4)
+        assert torch.isnan(states[1][0]).all() and torch.isnan(states[1][2]).all(), "another request's slot was written"
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_the_delta_rule_of_unequal_requests_in_one_batch(backend):
+    """Three steps of four requests of unequal lengths (single tokens first, as the batch orders them), on slots in
+    another order than the requests; one request ends and another takes its slot."""
+    k, dev = _kernels(backend)
+    shape, eps = (4, 2, 12, 8, 3), 1e-6
+    w = _delta_weights(shape, 21, torch.float32)
+    lens = {"a": 30, "b": 3, "c": 55, "d": 17, "e": 26}
+    inputs = {r: _delta_inputs(shape, n, 30 + i, torch.float32) for i, (r, n) in enumerate(lens.items())}
+    want = {r: _plain_delta(shape, w, inputs[r], eps) for r in lens}
+    states = _new_states(dev, 4, shape)
+    slot = {"a": 2, "b": 0, "c": 3, "d": 1, "e": 0}
+    steps = [[("b", 0, 1), ("a", 0, 30), ("c", 0, 20), ("d", 0, 2)],
+             [("b", 1, 1), ("d", 2, 1), ("c", 20, 33)],
+             [("b", 2, 1), ("c", 53, 1), ("d", 3, 14)],
+             [("c", 54, 1), ("e", 0, 26)]]                              # e takes b's slot, which holds b's last state
+    got = {r: [] for r in lens}
+    for step in steps:
+        part = tuple(torch.cat([inputs[r][i][s:s + n] for r, s, n in step]) for i in range(3))
+        out = _run_delta(k, dev, shape, w, part, eps, states, [n for _, _, n in step], [s for _, s, _ in step],
+                         [slot[r] for r, _, _ in step])
+        row = 0
+        for r, s, n in step:
+            got[r].append(out[row:row + n])
+            row += n
+    for r in lens:
+        _close(torch.cat(got[r]), want[r], torch.float32, r, 1e-4)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_the_delta_rule_keeps_and_forgets_by_its_decay(backend):
+    """A head whose decay is next to one still reads out, hundreds of tokens later, the value written for a key that
+    no later key touched; a head that forgets fast does not.  The state is float32: the far value comes back to 1e-4."""
+    k, dev = _kernels(backend)
+    shape, eps, T = (2, 1, 16, 8, 1), 1e-6, 400
+    heads, kv_heads, dim, vdim, taps = shape
+    w = _delta_weights(shape, 5, torch.float32, slow=0)
+    w["A_log"][1] = 1.0
+    w["conv"][:] = 1.0                                       # one tap of weight 1: the convolution passes its input
+    C = 2 * dim + heads * vdim
+    proj = torch.zeros((T, C + heads))
+    big = 30.0                                               # silu(30) = 30; unit norm makes q and k axis vectors
+    proj[:, :dim] = -30.0                                    # silu(-30) ~ 0
+    proj[:, dim:2 * dim] = -30.0
+    proj[0, dim + 3] = big                                   # token 0 writes at key axis 3
+    proj[1:, dim + 5] = big                                  # every later token writes at key axis 5
+    proj[-1, 3] = big                                        # the last token asks for axis 3
+    proj[:-1, 5] = big
+    g = torch.Generator().manual_seed(9)
+    proj[:, 2 * dim:C] = torch.randn((T, heads * vdim), generator=g)
+    proj[:, C:] = 30.0                                       # beta = 1: a write replaces what its key read
+    decay_in = torch.zeros((T, heads * dim))
+    gate_in = torch.full((T, heads * vdim), 30.0)            # gate = 1
+    w["norm"][:] = 1.0
+    w["dt_bias"][:] = 0.0
+    inputs = (proj, decay_in, gate_in)
+    want = _plain_delta(shape, w, inputs, eps)
+    for portions in ([T], [T - 1, 1], [150, 249, 1]):
+        states = _new_states(dev, 1, shape)
+        outs, pos = [], 0
+        for n in portions:
+            outs.append(_run_delta(k, dev, shape, w, tuple(t[pos:pos + n] for t in inputs), eps, states, [n], [pos], [0]))
+            pos += n
+        got = torch.cat(outs).cpu()
+        _close(got, want, torch.float32, portions, 1e-4)
+        v0 = plain.silu(proj[0, 2 * dim:2 * dim + vdim].double())
+        last = got[-1, :vdim].double()
+        assert float((last - plain.unit_mean(v0, eps)).abs().max()) < 1e-3, "the slow head lost token 0"
+        assert float(want[-1, vdim:].abs().max()) < 1e-3 and float(got[-1, vdim:].abs().max()) < 1e-3, "the fast head kept it"
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_the_convolution_reads_exactly_its_taps(backend):
+    """An impulse in q's input: it shows in the outputs of the next taps - 1 tokens and no further, also over a
+    portion's edge."""
+    k, dev = _kernels(backend)
+    shape, eps, T = (1, 1, 8, 8, 4), 1e-6, 12
+    w = _delta_weights(shape, 5, torch.float32)
+    base = _delta_inputs(shape, T, 6, torch.float32)
+    bumped = tuple(t.clone() for t in base)
+    bumped[0][4, 2 * 8 + 3] += 5.0                             # v's channel 3 at token 4: v enters u only, and S from then on
+    for portions in ([T], [5, 7], [6, 6], [4, 1, 1, 1, 1, 4]):
+        outs = []
+        for inputs in (base, bumped):
+            states = _new_states(dev, 1, shape)
+            got, pos = [], 0
+            for n in portions:
+                got.append(_run_delta(k, dev, shape, w, tuple(t[pos:pos + n] for t in inputs), eps, states, [n], [pos], [0]))
+                pos += n
+            outs.append(torch.cat(got).cpu())
+        assert torch.equal(outs[0][:4], outs[1][:4]) and not torch.equal(outs[0][4], outs[1][4])
+        _close(outs[1], _plain_delta(shape, w, bumped, eps), torch.float32, portions, 1e-4)
+
+
+# ------------------------------------------------------------------------------ the model through the step function
+def _runner(name, backend, dtype, pages, max_requests=4):
+    kernels, dev = _kernels(backend, torch.float32 if dtype == "float32" else torch.bfloat16)
+    return H.make_runner(K.model_folder(name, dtype), dtype, K.CONFIGS[name]["page"], pages, device=dev,
+                         kernels=kernels, max_requests=max_requests)
+
+
+MODEL_TOL = {"float32": 1e-4, "bfloat16": 6e-2}
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
+def test_every_cutting_gives_the_plain_logits(backend, name):
+    c = K.CONFIGS[name]
+    n = 70 if (backend, name) == ("cpu", "b") else 110
+    toks = H.random_tokens(c["cfg"].vocab, n, 1)
+    want = K.plain_logits(K.model_folder(name), toks)
+    r = _runner(name, backend, "float32", 40)
+    windows = {(l.mixer.window, l.mixer.keep_first if l.mixer.window else 0) for l in c["cfg"].layers if l.kind == "attention"}
+    assert len(r.cache.groups) == len(windows) and r.cache.slots.num_slots == 4
+    for portions in (H.whole(n), H.last_one_by_one(n, 45), H.changing_portions(n, 2), [1] * 3 + [2] * 10 + [n - 23]):
+        got = H.run_portions(r, "x", toks, portions)
+        assert K.err(got, want) < MODEL_TOL["float32"], portions
+    assert all(pool.num_free == 40 for pool in r.cache.pools)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["a", "b", "d"])
+def test_bfloat16_follows_the_plain_logits_under_every_cutting(name):
+    c = K.CONFIGS[name]
+    n = 130
+    toks = H.random_tokens(c["cfg"].vocab, n, 3)
+    want = K.plain_logits(K.model_folder(name, "bfloat16"), toks)
+    r = _runner(name, "hip", "bfloat16", 40)
+    for portions in (H.whole(n), H.last_one_by_one(n, 40), H.changing_portions(n, 4)):
+        e = K.errors(H.run_portions(r, "x", toks, portions), want)
+        # rounding may give a token another expert where two logits lie close: few positions, none far off
+        assert float(e.median()) < MODEL_TOL["bfloat16"] / 2 and float((e > MODEL_TOL["bfloat16"]).float().mean()) <= 0.05 \
+            and float(e.max()) < 0.6, (portions, float(e.median()), float(e.max()))
+
+
+@pytest.mark.gpu
+def test_a_larger_model_over_long_prompts():
+    """Six hundred tokens through a model with windows over several pages, seventy kept positions and delta-rule heads
+    of up to 128 channels: whole, in changing portions, and its last tokens one by one."""
+    name = "e"
+    c = K.CONFIGS[name]
+    n = 600
+    toks = H.random_tokens(c["cfg"].vocab, n, 17)
+    want = K.plain_logits(K.model_folder(name), toks)
+    r = _runner(name, "hip", "float32", 12)
+    assert len(r.cache.groups) == 2
+    for portions in (H.whole(n), H.changing_portions(n, 5), H.last_one_by_one(n, 180)):
+        assert K.err(H.run_portions(r, "x", toks, portions), want) < MODEL_TOL["float32"], portions[:4]
+    assert all(pool.num_free == 12 for pool in r.cache.pools)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_the_first_tokens_of_a_sequence(backend):
+    for name in ("a", "c"):
+        c = K.CONFIGS[name]
+        r = _runner(name, backend, "float32", 8)
+        for n in (1, 2, 3, 5):
+            toks = H.random_tokens(c["cfg"].vocab, n, 40 + n)
+            want = K.plain_logits(K.model_folder(name), toks)
+            for portions in ([n], [1] * n):
+                assert K.err(H.run_portions(r, "x", toks, portions), want) < MODEL_TOL["float32"], (name, n, portions)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", ["a", "c"])
+def test_long_decoding(backend, name):
+    # one prompt token, then 170 tokens one by one: windows pass over decoded tokens, the state is carried all the way
+    c = K.CONFIGS[name]
+    n = 171
+    toks = H.random_tokens(c["cfg"].vocab, n, 5)
+    want = K.plain_logits(K.model_folder(name), toks)
+    r = _runner(name, backend, "float32", 48)
+    assert K.err(H.run_portions(r, "x", toks, [1] * n), want) < MODEL_TOL["float32"]
+    if name == "a":
+        # a window's group holds the pages of its window and of the kept first positions only
+        r.cache.admit("y")
+        for pos in range(n):
+            r.cache.reserve("y", pos + 1)
+        by_window = {g.window: sum(1 for p in t if p >= 0) for g, t in zip(r.cache.groups, r.cache.requests["y"].tables)}
+        assert by_window[10] <= 3 + 1 and by_window[21] <= 4, by_window
+        r.cache.release("y")
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", ["a", "d"])
+def test_mixed_batches_on_pages_and_slots_that_are_used_again(backend, name):
+    c = K.CONFIGS[name]
+    lens = {"r0": 60, "r1": 41, "r2": 77, "r3": 1, "r4": 35, "r5": 52, "r6": 66, "r7": 2}
+    reqs = {r: H.random_tokens(c["cfg"].vocab, n, i) for i, (r, n) in enumerate(lens.items())}
+    pages = 192 // c["page"]                   # 192 tokens of cache and three state slots for 334 tokens of eight requests
+    r = _runner(name, backend, "float32", pages, max_requests=3)
+    got = H.run_mixed(r, reqs, seed=3, max_live=3)
+    for rid, toks in reqs.items():
+        assert K.err(got[rid], K.plain_logits(K.model_folder(name), toks)) < MODEL_TOL["float32"], rid
+    assert all(pool.num_free == pages for pool in r.cache.pools) and r.cache.slots.num_free == 3
+    # each request alone gives what it gave in the batches
+    alone = _runner(name, backend, "float32", pages, max_requests=1)
+    for rid in ("r1", "r3", "r6"):
+        one = H.run_portions(alone, rid, reqs[rid], [len(reqs[rid])])
+        assert K.err(got[rid], one) < 1e-5, rid
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_the_residual_stream_after_every_layer(backend):
+    """Layer by layer: the float32 stream after a layer is the plain implementation's.  The stream takes a layer's
+    last addend inside the norm that follows, so it is read where that norm leaves it."""
+    name = "a"
+    c = K.CONFIGS[name]
+    toks = H.random_tokens(c["cfg"].vocab, 37, 9)
+    cfg, w = K.plain_model(K.model_folder(name))
+    _, streams = plain.forward(cfg, w, toks, return_layers=True)
+    r = _runner(name, backend, "float32", 8)
+    seen = []
+    inner = r.kernels.stream_rms_norm
+
+    def spy(addends, residual, *a, **kw):
+        y, res = inner(addends, residual, *a, **kw)
+        seen.append(res.detach().float().cpu().clone())
+        return y, res
+    r.kernels.stream_rms_norm = spy
+    try:
+        H.run_portions(r, "x", toks, [len(toks)])
+    finally:
+        del r.kernels.stream_rms_norm
+    # the stream is seen by every pre-norm: two a layer with a feed-forward, one without, and the final one
+    at, ends = 0, []
+    for layer in cfg["layers"]:
+        at += 2 if layer.get("mlp") else 1
+        ends.append(at)                                   # the norm that first sees the stream after this layer
+    assert len(seen) == at + 1
+    for i, want in enumerate(streams):
+        assert float((seen[ends[i]].double() - want).abs().max() / want.abs().max()) < 2e-5, i
+
+
+# ------------------------------------------------------------------------------ the engine
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("schedule", ["prefill_first", "mixed"])
+def test_greedy_generation_through_the_engine(backend, schedule):
+    name = "d"
+    c = K.CONFIGS[name]
+    kernels, dev = _kernels(backend)
+    folder = K.model_folder(name)
+    prompts = [H.random_tokens(c["cfg"].vocab, n, 60 + n) for n in (3, 30, 1, 47, 18)]
+    # few pages, three request slots and portions of at most 16 tokens: prompts are cut, requests wait
+    llm = LLM(folder, kernels=kernels, device=dev, dtype="float32", kvcache_block_size=c["page"], num_kvcache_blocks=10,
+              max_num_batched_tokens=16, max_num_seqs=3, schedule=schedule, max_model_len=128)
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True), use_tqdm=False)
+    cfg, w = K.plain_model(folder)
+    for p, o in zip(prompts, outs):
+        assert o["token_ids"] == plain.greedy_generate(cfg, w, p, 10), len(p)
+    assert llm.runner.cache.slots.num_free == 3 and all(pool.num_free == 10 for pool in llm.runner.cache.pools)
+
+
+@pytest.mark.gpu
+def test_generation_in_bfloat16_with_captured_steps_and_bursts():
+    name = "b"
+    c = K.CONFIGS[name]
+    folder = K.model_folder(name, "bfloat16")
+    prompts = [H.random_tokens(c["cfg"].vocab, n, 80 + n) for n in (5, 40, 90, 17)]
+    sp = SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True)
+    common = dict(dtype="bfloat16", kvcache_block_size=c["page"], num_kvcache_blocks=24, max_num_seqs=4, max_model_len=256)
+    eager = LLM(folder, enforce_eager=True, **common).generate(prompts, sp, use_tqdm=False)
+    graphs = LLM(folder, decode_burst=8, **common)
+    assert graphs.runner._graph_max_batch, "the delta rule reads the step's metadata on the device: its steps are captured"
+    fast = graphs.generate(prompts, sp, use_tqdm=False)
+    for a, b in zip(eager, fast):
+        assert a["token_ids"] == b["token_ids"]
+
+
+@pytest.mark.gpu
+def test_trace_replay_of_a_model_folder(tmp_path):
+    """bin/trace_run as a process on a Kirisun folder: portions, single tokens and a second request that takes the
+    first one's pages and slot."""
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    name = "d"
+    c = K.CONFIGS[name]
+    folder = K.model_folder(name)
+    a, b = H.random_tokens(c["cfg"].vocab, 50, 1), H.random_tokens(c["cfg"].vocab, 70, 2)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:33], "want": [0, 32]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[33:34], "want": [0]}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[34:], "want": [15]}, {"id": "b", "tokens": b[:2], "want": []}], "end": ["a"]},
+             {"step": 3, "entries": [{"id": "b", "tokens": b[2:], "want": [67]}], "end": ["b"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+                           "--out", str(out), "--max-tokens", "128", "--page-size", str(c["page"])],
+                          input="\n".join(json.dumps(s) for s in steps) + "\n", text=True, capture_output=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+    wa, wb = K.plain_logits(folder, a), K.plain_logits(folder, b)
+    V = c["cfg"].vocab
+    read = lambda i: torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, V))
+    assert K.err(read(0), wa[[0, 32]]) < 1e-4 and K.err(read(1), wa[[33]]) < 1e-4
+    assert K.err(read(2), wa[[49]]) < 1e-4 and K.err(read(3), wb[[69]]) < 1e-4
