@@ -70,6 +70,8 @@ def parse_args():
     ap.add_argument("--design", default=None, choices=["nozurax", "mafarax", "kirisun"],
                     help="measure this design beside Qwen3 at equal layer sizes instead of the default workload")
     ap.add_argument("--design-sizes", default="1024,2048,4096", help="model widths of the --design measurement")
+    ap.add_argument("--design-alone", action="store_true", help="the --design measurement without the models beside it "
+                                                                "(a profiler's run then holds that design's kernels only)")
     return ap.parse_args()
 
 
@@ -141,6 +143,8 @@ def design_run(args):
     for width in [int(w) for w in args.design_sizes.split(",") if w]:
         out[width] = {}
         for name, config_json in design_configs(width, layers, args.dtype, args.design).items():
+            if args.design_alone and name != args.design:
+                continue
             arch = architecture_of(config_json)
             model = Model(arch.build_spec(arch.parse_config(config_json)), kernels, device, dtype)
             fill_random_(model, args.seed)

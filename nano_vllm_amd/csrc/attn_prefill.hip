@@ -94,8 +94,8 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
                     const int32_t* __restrict__ block_tables, int table_stride,
                     const int32_t* __restrict__ cu_seqlens_q, const int32_t* __restrict__ kv_lens,
                     const int32_t* __restrict__ tiles, int num_tiles, int paired, int num_q_heads, int num_kv_heads,
-                    int page_size, float scale, int window, int key_chunk, const float* __restrict__ sinks,
-                    int32_t* error_flag) {
+                    int page_size, float scale, int window, int key_chunk, int keep_first, float softcap,
+                    const float* __restrict__ sinks, int32_t* error_flag) {
     constexpr int DC = D / 16;            // 16-channel steps of the first product
     constexpr int MT = D / 32;            // 32-channel tiles of the output
     constexpr int KR = D / 8;             // 16-byte pieces of a K row (one key)
@@ -160,6 +160,13 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     const int first_any = nva_first_key(start + q0, window, key_chunk);
     const int kb_lo = first_any & ~(PF_BN - 1);
     const int kb_hi = last_pos + 1;                   // exclusive
+    // Kept first positions (with a window): keys below `keep` stay visible to every row.  Those before the first
+    // tile of the window's keys are read through tiles of their own, which run first: tile numbers below kb_lo
+    // stand for them (v_lo: the first), and real() says where a tile's keys begin.
+    const int keep = window > 0 ? keep_first : 0;
+    const int pre_keys = min(keep, kb_lo);
+    const int v_lo = kb_lo - (pre_keys + PF_BN - 1) / PF_BN * PF_BN;
+    auto real = [&](int v) __attribute__((always_inline)) { return v >= kb_lo ? v : v - v_lo; };
 
     // ---- Q: column = query row, lane half h holds channels 16c + 8h .. + 7
     bf16x8 qf[DC];
@@ -199,6 +206,17 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
         if (page < 0 && page_lo + i >= first_any / page_size && error_flag) atomicOr(error_flag, 2);
         table_s[i] = max(page, 0);
     }
+    // the pages of the kept first positions that lie before those: behind them in the buffer
+    const int kept_pages = min((pre_keys + page_size - 1) / page_size, page_lo);
+    for (int i = threadIdx.x; i < kept_pages; i += SETS * SET_THREADS) {
+        const int page = table[i];
+        if (page < 0 && error_flag) atomicOr(error_flag, 2);
+        table_s[num_pages + i] = max(page, 0);
+    }
+    auto page_of = [&](int key) __attribute__((always_inline)) {
+        const int p = key / page_size;
+        return table_s[p >= page_lo ? p - page_lo : num_pages + p];
+    };
     // the Q loads are done before the tiles' loads are counted
     wait_loads_but<0>();
     barrier();
@@ -251,7 +269,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     // key index and what V holds for them is cleared in LDS); a tile past the last is the last again.
     auto load_in_page = [&](const __bf16* cache, int kb, const uint32_t* off, uint32_t lds) __attribute__((always_inline)) {
         kb = min(kb, after_last);
-        const int page = __builtin_amdgcn_readfirstlane(table_s[kb / page_size - page_lo]);
+        const int page = __builtin_amdgcn_readfirstlane(page_of(kb));
         load_fast(cache, page, kb % page_size, off, lds);
     };
     auto load_k_any = [&](int kb, int buf) __attribute__((always_inline)) {
@@ -261,8 +279,10 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
         for (int i = 0; i < PIECES; ++i) {
             const int n = (PF_WAVES * i + wave) * NVA_WAVE + lane;
             const int r = n / KR, piece = SwK::slot(r, n % KR);
-            const int key = min(max(kb + r, first_any), last_key);
-            const int page = table_s[key / page_size - page_lo];
+            int key = kb + r;
+            if (key >= keep) key = max(key, first_any);
+            key = min(key, last_key);
+            const int page = page_of(key);
             load_to_lds(k_cache + (((int64_t)page * num_kv_heads + kvh) * page_size + key % page_size) * D + piece * 8,
                         dst + i * LOAD_BYTES);
         }
@@ -274,8 +294,10 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
         for (int i = 0; i < PIECES; ++i) {
             const int n = (PF_WAVES * i + wave) * NVA_WAVE + lane;
             const int d = n / VR, group = SwV::slot(d, n % VR);
-            const int key0 = min(max(kb + group * 8, first_any & ~7), last_key & ~7);
-            const int page = table_s[key0 / page_size - page_lo];
+            int key0 = kb + group * 8;
+            if (key0 >= keep) key0 = max(key0, first_any & ~7);
+            key0 = min(key0, last_key & ~7);
+            const int page = page_of(key0);
             load_to_lds(v_cache + ((int64_t)page * num_kv_heads + kvh) * D * (int64_t)page_size +
                             nva_v_offset(key0 % page_size, d, D, vt),
                         dst + i * LOAD_BYTES);
@@ -294,7 +316,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
                 bf16x8 v = *reinterpret_cast<bf16x8*>(tile_v + n * 8);
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    if (key0 + e >= kb_hi || key0 + e < first_any) v[e] = (__bf16)0.f;
+                    if (key0 + e >= kb_hi || (key0 + e < first_any && key0 + e >= keep)) v[e] = (__bf16)0.f;
                 *reinterpret_cast<bf16x8*>(tile_v + n * 8) = v;
             }
         }
@@ -308,15 +330,26 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     // this lane: query `col`; register e of tile kt is key kb + 32*kt + 16*(e/8) + 8*h + e%8.
     // The maximum is taken of the raw scores (scale > 0) and the scale folded, with log2(e),
     // into the exponent: p = 2^((s - m) * scale * log2 e), one fused multiply-add per score.
+    // A cap on the scores: x = scale * s becomes cap * tanh(x / cap); in the raw scores' units, which the maximum and
+    // the exponent keep, s <- (cap / scale) * tanh(s * scale / cap), with tanh(y) = 1 - 2 / (1 + e^(2 y)).
+    const bool capped = softcap > 0.f;
+    const float cap_in = capped ? 2.f * 1.4426950408889634f * scale / softcap : 0.f, cap_out = capped ? softcap / scale : 0.f;
     auto softmax = [&](int kb, auto masked_tag) __attribute__((always_inline)) {
         float m_new = m_run;
+        if (capped) {
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    s[kt][e] = cap_out - 2.f * cap_out * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(s[kt][e] * cap_in));
+        }
         if (decltype(masked_tag)::value) {
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int key = kb + 32 * kt + 16 * (e >> 3) + 8 * h + (e & 7);
-                    if (key > pos || key < first_row) s[kt][e] = -INFINITY;
+                    if (key > pos || (key < first_row && key >= keep)) s[kt][e] = -INFINITY;
                 }
         }
 #pragma unroll
@@ -433,10 +466,11 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
         if (fast_pages) load_in_page(v_cache, kb, v_off, lds_wave + (2 + b) * 2 * TILE);
         else load_v_any(kb, b);
     };
-    auto round = [&](int kb, auto masked_tag) __attribute__((always_inline)) {
+    auto round = [&](int tile, auto masked_tag) __attribute__((always_inline)) {
+        const int kb = real(tile);
         if (active) softmax(kb, masked_tag);
-        load_k(kb + 2 * STEP, buf);
-        load_v(kb + STEP, buf ^ 1);
+        load_k(real(tile + 2 * STEP), buf);
+        load_v(real(tile + STEP), buf ^ 1);
         wait_loads_but<2 * PIECES>();
         if (decltype(masked_tag)::value && (kb < first_any || kb + PF_BN > kb_hi)) clear_v_outside(kb, buf);
         products();
@@ -464,12 +498,12 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
         next_page = page, next_entry = entry, next_kip = kip;
         products();
     };
-    const int rounds = ((kb_hi - kb_lo + PF_BN - 1) / PF_BN + SETS - 1) / SETS;
+    const int rounds = ((kb_hi - v_lo + PF_BN - 1) / PF_BN + SETS - 1) / SETS;
     if (SETS > 1 && set == 1) barrier();
-    int kb = kb_lo + set * PF_BN;
-    load_k(kb, 0);
-    load_k(kb + STEP, 1);
-    load_v(kb, 0);
+    int kb = v_lo + set * PF_BN;                     // a tile number: real(kb) is where its keys begin
+    load_k(real(kb), 0);
+    load_k(real(kb + STEP), 1);
+    load_v(real(kb), 0);
     wait_loads_but<2 * PIECES>();
     barrier();
     if (active) products_of(0, 0, No());
@@ -543,7 +577,8 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
                                      int table_stride, const int32_t* cu_seqlens_q, const int32_t* kv_lens,
                                      const int32_t* tiles, int64_t num_tiles, int num_q_heads,
                                      int num_kv_heads, int head_dim, int page_size, float scale, int window, int chunk,
-                                     const float* sinks, int32_t* error_flag, hipStream_t stream) {
+                                     int keep_first, float softcap, const float* sinks, int32_t* error_flag,
+                                     hipStream_t stream) {
     if (num_tiles == 0) return 0;
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads)
         return nva_fail("attn_prefill: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
@@ -559,6 +594,8 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
     }
     const int G = num_q_heads / num_kv_heads;
     const int64_t grid_y = (int64_t)num_kv_heads * ((G + PF_WAVES - 1) / PF_WAVES);
+    if (keep_first < 0 || !(softcap >= 0.f) || !(softcap <= 3.0e38f))
+        return nva_fail("attn_prefill: bad kept positions %d or cap %g", keep_first, (double)softcap);
     if (!tiles || num_tiles < 0 || num_tiles * grid_y > 0x7fffffff || window < 0 || chunk < 0 || table_stride <= 0)
         return nva_fail("attn_prefill: bad sizes (tiles %lld, heads %lld)", (long long)num_tiles, (long long)grid_y);
     if (table_stride > 4096) {
@@ -583,7 +620,7 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
                        (const __bf16*)q, q_stride, (__bf16*)out, out_stride, (const __bf16*)k_cache,                 \
                        (const __bf16*)v_cache, block_tables, table_stride, cu_seqlens_q, kv_lens, tiles,             \
                        (int)num_tiles, SS == 1 && PF_WAVES_PER_SIMD(DD) == 2 && total <= 2 * cus ? (int)total : 0,   \
-                       num_q_heads, num_kv_heads, page_size, scale, window, chunk, sinks, error_flag)
+                       num_q_heads, num_kv_heads, page_size, scale, window, chunk, keep_first, softcap, sinks, error_flag)
 #define LAUNCH(DD)                                                                                                 \
     do {                                                                                                           \
         if (PF_WAVES_PER_SIMD(DD) == 2 && two_sets) LAUNCH_SETS(DD, PF_WAVES_PER_SIMD(DD));                         \

@@ -15,17 +15,20 @@
 // Everything after the projections is float whatever the element type (the convolutions' sums, the unit norms,
 // softplus and the exponentials by the accurate routines, the state, the read-out, the norm and the gate); y is
 // rounded once.  A token's sums run in an order that neither the portion's cut nor the batch changes: the
-// recurrence goes token by token, a thread holding one column of S in registers.
+// recurrence goes token by token, 8 lanes holding one column of S in registers.
 //
 //   delta_prepare     one workgroup a token: the convolutions, unit norms, beta and the decay, written as floats
 //   delta_keep        the request's new kept inputs (its last taps - 1), after delta_prepare has read the old ones
-//   delta_scan        one wave per (request, head, 64 columns of S): the recurrence over the portion's tokens, the
-//                     tokens' q, k and a staged in LDS a batch at a time, v and beta asked for a batch ahead
+//   delta_scan        four waves per (request, head, 32 columns of S), 8 lanes a column: the recurrence over the
+//                     portion's tokens, the tokens' q, k, a and beta staged in LDS a batch at a time in two buffers,
+//                     v asked for a batch ahead
 //   delta_finish      one wave per (token, head): the norm and the gate
 #include "common.h"
 
 #define DELTA_MAX_TAPS 16
 #define DELTA_BATCH 8            // tokens whose q, k and a lie in LDS at a time
+#define DELTA_THREADS 256        // of the recurrence's workgroup: four waves
+#define DELTA_COLS 32            // columns of S a workgroup holds, 8 lanes a column
 
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -101,45 +104,88 @@ delta_keep_kernel(const T* __restrict__ proj, int64_t stride, float* __restrict_
     for (int i = 0; i < taps - 1; ++i) kept[i] = fresh[i];
 }
 
-// One wave per (request, head, 64 columns of S).  A thread holds its column's DMAX rows (rows beyond D: zeros, with
-// q, k and a staged as zeros).  Per token, in this order: S <- a S, u = beta (v - S^T k), S <- S + k u, o = S^T q; the
-// two sums over the rows run as four chains each, in an order that depends on D alone.
+// The sum of x over the 8 neighbouring lanes that share a column of S (lanes 8c .. 8c + 7): two exchanges inside
+// the quads, then one between the two quads, which by then hold one value each.
+__device__ __forceinline__ float delta_sum8(float x) {
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0xB1, 0xF, 0xF, true));     // lanes 1 0 3 2
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x4E, 0xF, 0xF, true));     // lanes 2 3 0 1
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x141, 0xF, 0xF, true));    // lanes 7 .. 0 of each 8
+    return x;
+}
+
+// One workgroup of four waves per (request, head, 32 columns of S).  A column's DMAX rows (rows beyond D: zeros,
+// with q, k and a staged as zeros) lie in 8 neighbouring lanes: lane r of them holds the rows 4 (r + 8 j) .. + 3 for
+// j < DMAX / 32, so that the 8 lanes read 32 consecutive floats of a staged row at a time.  Per token, in this order:
+// S <- a S, u = beta (v - S^T k), S <- S + k u, o = S^T q; each of the two sums over the rows runs as four chains a
+// lane and then over the 8 lanes, in an order that depends on D alone.  The tokens' q, k, a and beta go through LDS,
+// a batch at a time in two buffers: the next batch is asked for before this one's sums and stored after them.
 template <int DMAX>
-__global__ void __launch_bounds__(NVA_WAVE)
+__global__ void __launch_bounds__(DELTA_THREADS)
 delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vf,
                   const float* __restrict__ decay, const float* __restrict__ beta, float* __restrict__ o_raw,
                   float* __restrict__ state, const int32_t* __restrict__ cu_seqlens_q,
                   const int32_t* __restrict__ seq_starts, const int32_t* __restrict__ state_slots, int heads,
                   int kv_heads, int dim, int vdim) {
-    __shared__ __attribute__((aligned(16))) float q_s[DELTA_BATCH][DMAX], k_s[DELTA_BATCH][DMAX], a_s[DELTA_BATCH][DMAX];
-    __shared__ float beta_s[DELTA_BATCH];
-    const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const int col = blockIdx.z * NVA_WAVE + lane;
+    constexpr int R4 = DMAX / 32;                                       // float4s of rows a lane holds
+    constexpr int STAGED = 3 * DELTA_BATCH * DMAX;                      // q, k, a of a batch
+    constexpr int NP = (STAGED + DELTA_THREADS - 1) / DELTA_THREADS;
+    __shared__ __attribute__((aligned(16))) float qka_s[2][3][DELTA_BATCH][DMAX];
+    __shared__ float beta_s[2][DELTA_BATCH];
+    const int seq = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int r = tid & 7;
+    const int col = blockIdx.z * DELTA_COLS + (tid >> 3);
     const bool live = col < vdim;
     const int g = h / (heads / kv_heads);
     const int begin = cu_seqlens_q[seq], n = cu_seqlens_q[seq + 1] - begin;
     const int qk = kv_heads * dim, vv = heads * vdim, hd = heads * dim;
     float* S_g = state + (((int64_t)state_slots[seq] * heads + h) * dim) * vdim + col;
-    float S[DMAX];
     const bool has_past = seq_starts[seq] > 0;
+    float S[4 * R4];
 #pragma unroll
-    for (int i = 0; i < DMAX; ++i) S[i] = has_past && live && i < dim ? S_g[(int64_t)i * vdim] : 0.f;
+    for (int j = 0; j < R4; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = 4 * (r + 8 * j) + e;
+            S[4 * j + e] = has_past && live && row < dim ? S_g[(int64_t)row * vdim] : 0.f;
+        }
 
+    // a batch's q, k, a (and beta) from global memory into registers, and from there into one of the two buffers
+    float pre[NP], pre_beta = 0.f;
+    auto ask = [&](int t0) __attribute__((always_inline)) {
+        const int nb = min(DELTA_BATCH, n - t0);
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            const int e = i * DELTA_THREADS + tid;
+            const int which = e / (DELTA_BATCH * DMAX), b = (e / DMAX) % DELTA_BATCH, d = e % DMAX;
+            float x = 0.f;
+            if (e < STAGED && b < nb && d < dim) {
+                const int64_t tok = begin + t0 + b;
+                x = which == 0 ? qn[tok * qk + g * dim + d] : which == 1 ? kn[tok * qk + g * dim + d] : decay[tok * hd + h * dim + d];
+            }
+            pre[i] = x;
+        }
+        pre_beta = tid < nb ? beta[(int64_t)(begin + t0 + tid) * heads + h] : 0.f;
+    };
+    auto put = [&](int buf) __attribute__((always_inline)) {
+        float* flat = &qka_s[buf][0][0][0];
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            const int e = i * DELTA_THREADS + tid;
+            if (e < STAGED) flat[e] = pre[i];
+        }
+        if (tid < DELTA_BATCH) beta_s[buf][tid] = pre_beta;
+    };
     float v_next[DELTA_BATCH];
 #pragma unroll
     for (int b = 0; b < DELTA_BATCH; ++b) v_next[b] = live && b < n ? vf[(int64_t)(begin + b) * vv + h * vdim + col] : 0.f;
-    for (int t0 = 0; t0 < n; t0 += DELTA_BATCH) {
+    ask(0);
+    put(0);
+    __syncthreads();
+    int buf = 0;
+    for (int t0 = 0; t0 < n; t0 += DELTA_BATCH, buf ^= 1) {
         const int nb = min(DELTA_BATCH, n - t0);
-        __syncthreads();                                               // the batch before is done with
-        for (int i = lane; i < DELTA_BATCH * DMAX; i += NVA_WAVE) {
-            const int b = i / DMAX, d = i % DMAX;
-            const bool ok = b < nb && d < dim;
-            const int64_t tok = begin + t0 + b;
-            q_s[b][d] = ok ? qn[tok * qk + g * dim + d] : 0.f;
-            k_s[b][d] = ok ? kn[tok * qk + g * dim + d] : 0.f;
-            a_s[b][d] = ok ? decay[tok * hd + h * dim + d] : 0.f;
-        }
-        if (lane < DELTA_BATCH) beta_s[lane] = lane < nb ? beta[(int64_t)(begin + t0 + lane) * heads + h] : 0.f;
+        const bool more = t0 + DELTA_BATCH < n;
+        if (more) ask(t0 + DELTA_BATCH);
         float v_now[DELTA_BATCH];
 #pragma unroll
         for (int b = 0; b < DELTA_BATCH; ++b) {
@@ -147,34 +193,44 @@ delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn, co
             const int tn = t0 + DELTA_BATCH + b;                        // the batch after: asked for now
             v_next[b] = live && tn < n ? vf[(int64_t)(begin + tn) * vv + h * vdim + col] : 0.f;
         }
-        __syncthreads();
 #pragma unroll
         for (int b = 0; b < DELTA_BATCH; ++b) {
             if (b >= nb) break;
+            const float* q_row = qka_s[buf][0][b];
+            const float* k_row = qka_s[buf][1][b];
+            const float* a_row = qka_s[buf][2][b];
+            float4 kr[R4];
             float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
 #pragma unroll
-            for (int i = 0; i < DMAX; i += 4) {
-                const float4 a = *reinterpret_cast<const float4*>(&a_s[b][i]);
-                const float4 k = *reinterpret_cast<const float4*>(&k_s[b][i]);
-                S[i] *= a.x; S[i + 1] *= a.y; S[i + 2] *= a.z; S[i + 3] *= a.w;
-                d0 += S[i] * k.x; d1 += S[i + 1] * k.y; d2 += S[i + 2] * k.z; d3 += S[i + 3] * k.w;
+            for (int j = 0; j < R4; ++j) {
+                const float4 a = *reinterpret_cast<const float4*>(a_row + 4 * (r + 8 * j));
+                const float4 k = kr[j] = *reinterpret_cast<const float4*>(k_row + 4 * (r + 8 * j));
+                S[4 * j] *= a.x; S[4 * j + 1] *= a.y; S[4 * j + 2] *= a.z; S[4 * j + 3] *= a.w;
+                d0 += S[4 * j] * k.x; d1 += S[4 * j + 1] * k.y; d2 += S[4 * j + 2] * k.z; d3 += S[4 * j + 3] * k.w;
             }
-            const float u = beta_s[b] * (v_now[b] - ((d0 + d1) + (d2 + d3)));
+            const float u = beta_s[buf][b] * (v_now[b] - delta_sum8((d0 + d1) + (d2 + d3)));
             float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
-            for (int i = 0; i < DMAX; i += 4) {
-                const float4 k = *reinterpret_cast<const float4*>(&k_s[b][i]);
-                const float4 q = *reinterpret_cast<const float4*>(&q_s[b][i]);
-                S[i] += k.x * u; S[i + 1] += k.y * u; S[i + 2] += k.z * u; S[i + 3] += k.w * u;
-                o0 += S[i] * q.x; o1 += S[i + 1] * q.y; o2 += S[i + 2] * q.z; o3 += S[i + 3] * q.w;
+            for (int j = 0; j < R4; ++j) {
+                const float4 k = kr[j];
+                const float4 q = *reinterpret_cast<const float4*>(q_row + 4 * (r + 8 * j));
+                S[4 * j] += k.x * u; S[4 * j + 1] += k.y * u; S[4 * j + 2] += k.z * u; S[4 * j + 3] += k.w * u;
+                o0 += S[4 * j] * q.x; o1 += S[4 * j + 1] * q.y; o2 += S[4 * j + 2] * q.z; o3 += S[4 * j + 3] * q.w;
             }
-            if (live) o_raw[(int64_t)(begin + t0 + b) * vv + h * vdim + col] = (o0 + o1) + (o2 + o3);
+            const float o = delta_sum8((o0 + o1) + (o2 + o3));
+            if (live && r == 0) o_raw[(int64_t)(begin + t0 + b) * vv + h * vdim + col] = o;
         }
+        if (more) put(buf ^ 1);
+        __syncthreads();                                                // the next batch is in; this one is done with
     }
     if (live) {
 #pragma unroll
-        for (int i = 0; i < DMAX; ++i)
-            if (i < dim) S_g[(int64_t)i * vdim] = S[i];
+        for (int j = 0; j < R4; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = 4 * (r + 8 * j) + e;
+                if (row < dim) S_g[(int64_t)row * vdim] = S[4 * j + e];
+            }
     }
 }
 
@@ -247,9 +303,9 @@ NVA_EXPORT int NVA_NAME(nva_channel_delta)(const void* proj, int64_t stride, con
                            (const elem_t*)proj, stride, conv_state, cu_seqlens_q, seq_starts, state_slots, channels, taps);
     }
     {
-        const dim3 grid((unsigned)seqs, (unsigned)heads, (vdim + NVA_WAVE - 1) / NVA_WAVE);
+        const dim3 grid((unsigned)seqs, (unsigned)heads, (vdim + DELTA_COLS - 1) / DELTA_COLS);
 #define DELTA_SCAN(DM)                                                                                                   \
-        hipLaunchKernelGGL(delta_scan_kernel<DM>, grid, dim3(NVA_WAVE), 0, stream, qn, kn, vf, decay, beta, o_raw, s_state, \
+        hipLaunchKernelGGL(delta_scan_kernel<DM>, grid, dim3(DELTA_THREADS), 0, stream, qn, kn, vf, decay, beta, o_raw, s_state, \
                            cu_seqlens_q, seq_starts, state_slots, heads, kv_heads, dim, vdim)
         if (dim <= 32) DELTA_SCAN(32); else if (dim <= 64) DELTA_SCAN(64); else if (dim <= 128) DELTA_SCAN(128); else DELTA_SCAN(256);
 #undef DELTA_SCAN

@@ -1279,14 +1279,15 @@ class HipKernels:
         keep = int(keep_first) if window and keep_first else 0
         if cap < 0.0 or keep < 0:
             raise KernelError("attention: a negative softcap or number of kept positions")
-        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and v_dim == head_dim \
-            and cap == 0.0 and keep == 0
-        if batch.num_decode > 0 and mfma and \
+        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and v_dim == head_dim
+        # (the decode kernel knows neither a cap on the scores nor kept first positions: such single tokens run the
+        # general kernel, the portions of prompts beside them the matrix-core prefill kernel all the same)
+        if batch.num_decode > 0 and mfma and cap == 0.0 and keep == 0 and \
                 self._decode_kernel_takes(num_heads // num_kv_heads, head_dim, page_size, q, qs, out, os_):
             start = batch.num_decode
             self._attention_decode(q, qs, out, os_, k_cache, v_cache, tables, batch, start, num_heads, num_kv_heads,
                                    head_dim, page_size, scale, window, sinks, chunk)
-        if start < tokens and mfma and start == batch.num_decode and \
+        if batch.num_decode < tokens and mfma and \
                 self._prefill_kernel_takes(head_dim, page_size, tables.shape[1], q, qs, out, os_):
             # portions of prompts: the matrix-core prefill kernel, one workgroup per 32 query rows
             tiles = self._prefill_tiles(batch, q.device)
@@ -1294,8 +1295,8 @@ class HipKernels:
                          _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.cu_seqlens_q), _p(batch.kv_lens),
                          _p(tiles), c_i64(tiles.shape[0]), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
-                         c_i32(chunk or 0), _p(sinks), _p(self.fault_flag), self._stream())
-            start = tokens
+                         c_i32(chunk or 0), c_i32(keep), c_f32(cap), _p(sinks), _p(self.fault_flag), self._stream())
+            tokens = batch.num_decode            # what is left: the single tokens before the portions, if any
         if self.tiled_general_attention and start <= batch.num_decode < tokens and not window and \
                 max(head_dim, v_dim) <= GENERAL_TILED_MAX_HEAD_DIM:
             # portions of prompts in float arithmetic: the per-token kernel's arithmetic, operation for

@@ -123,8 +123,11 @@ class Attention(Part):
     @property
     def kernel_modules(self):
         prepare = "qk_rownorm" if self.row_prepare else "rope"
-        if self.v_head_dim != self.head_dim or self.softcap is not None or self.keep_first:
-            return (prepare, "attn_generic") + (("rope",) if self.row_prepare and self.position_encoding else ())
+        rope = ("rope",) if self.row_prepare and self.position_encoding else ()
+        if self.v_head_dim != self.head_dim:
+            return (prepare, "attn_generic") + rope
+        if self.softcap is not None or self.keep_first:        # single tokens run the general kernel
+            return (prepare, "attn_generic", "attn_prefill") + rope
         return (prepare, "attn_generic", "attn_decode", "attn_prefill") + \
             (("rope",) if self.row_prepare and self.position_encoding else ())
 
