@@ -1365,7 +1365,8 @@ class HipKernels:
         orows, ow, os_ = _rows2d(out, "delta-rule output")
         if (orows, ow) != (tokens, vv) or out.dtype != proj.dtype:
             raise KernelError("channel_delta: output does not match")
-        scratch = torch.empty(tokens * (2 * qk + 2 * vv + hd + heads), dtype=torch.float32, device=proj.device)
+        dp = (dim + 3) // 4 * 4                         # rows of q, k and the decays are padded to whole float4s
+        scratch = torch.empty(tokens * ((2 * kv_heads + heads) * dp + 2 * vv + heads), dtype=torch.float32, device=proj.device)
         library.call("delta", _suffix(proj), "nva_channel_delta", _p(proj), c_i64(stride), _p(decay_in), _p(gate_in), c_i64(gs),
                      _p(scratch), _p(out), c_i64(os_), _p(s_state), _p(conv_state if taps > 1 else None), _p(batch.token_seq),
                      _p(batch.cu_seqlens_q), _p(batch.seq_starts), _p(batch.state_slots), c_i64(seqs), c_i64(tokens),
