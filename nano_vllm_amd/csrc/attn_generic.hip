@@ -38,7 +38,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
                                const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
                                int num_q_heads, int num_kv_heads, int head_dim, int v_dim, int page_size, float scale,
                                int window, int chunk, int keep_first, float softcap, const float* __restrict__ sinks,
-                               int32_t* error_flag) {
+                               float* __restrict__ part, int32_t* error_flag) {
     __shared__ float q_s[ATT_MAX_D];
     __shared__ float p_s[NVA_WAVE];
     __shared__ int64_t v_off_s[NVA_WAVE];
@@ -59,15 +59,26 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
     float acc[ATT_ACC];
 #pragma unroll
     for (int i = 0; i < ATT_ACC; ++i) acc[i] = 0.f;
-    float m_run = sinks ? sinks[h] : -INFINITY, l_run = sinks ? 1.f : 0.f;
+    // part: the token's keys are shared out, in blocks of 64, among the gridDim.z workgroups of this (token, head);
+    // each leaves its maximum, sum and unnormalised output there, and paged_attention_merge_kernel joins them.
+    // The sink joins in the first share.
+    const int share = blockIdx.z, shares = gridDim.z;
+    const bool with_sink = sinks && share == 0;
+    float m_run = with_sink ? sinks[h] : -INFINITY, l_run = with_sink ? 1.f : 0.f;
     const bool vec = head_dim % 8 == 0;
     const int vt = nva_v_tile(page_size);
 
     // the kept first positions that the window has passed, [0, kept_end), then the window (or chunk) up to pos
     const int kept_end = window > 0 && keep_first > 0 ? min(keep_first, first) : 0;
-    for (int part = kept_end > 0 ? 0 : 1; part < 2; ++part) {
-    const int lo = part == 0 ? 0 : first, hi = part == 0 ? kept_end - 1 : pos;
-    for (int base = part == 1 && chunk > 0 ? first / NVA_WAVE * NVA_WAVE : lo; base <= hi; base += NVA_WAVE) {
+    const int window_base = chunk > 0 ? first / NVA_WAVE * NVA_WAVE : first;
+    const int blocks = (kept_end + NVA_WAVE - 1) / NVA_WAVE + (pos - window_base) / NVA_WAVE + 1;
+    const int per_share = (blocks + shares - 1) / shares;
+    const int block_lo = share * per_share, block_hi = min(blocks, block_lo + per_share);
+    int block = 0;
+    for (int run = kept_end > 0 ? 0 : 1; run < 2; ++run) {
+    const int lo = run == 0 ? 0 : first, hi = run == 0 ? kept_end - 1 : pos;
+    for (int base = run == 1 ? window_base : lo; base <= hi; base += NVA_WAVE, ++block) {
+        if (block < block_lo || block >= block_hi) continue;
         const int j = base + lane;
         float s = -INFINITY;
         int64_t v_off = 0;
@@ -144,7 +155,51 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
         }
     }
     }
+    if (part) {
+        float* mine = part + ((t * num_q_heads + h) * shares + share) * (int64_t)(2 + v_dim);
+        if (lane == 0) mine[0] = m_run, mine[1] = l_run;
+#pragma unroll
+        for (int i = 0; i < ATT_ACC; ++i) {
+            const int d = lane + i * NVA_WAVE;
+            if (d < v_dim) mine[2 + d] = acc[i];
+        }
+        return;
+    }
     const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+    T* orow = out + t * out_stride + (int64_t)h * v_dim;
+#pragma unroll
+    for (int i = 0; i < ATT_ACC; ++i) {
+        const int d = lane + i * NVA_WAVE;
+        if (d < v_dim) orow[d] = from_float<T>(acc[i] * inv);
+    }
+}
+
+// One wave per (token, head): the shares' results joined, in the order of the shares.
+template <typename T>
+__global__ void __launch_bounds__(NVA_WAVE)
+paged_attention_merge_kernel(const float* __restrict__ part, int shares, T* __restrict__ out, int64_t out_stride,
+                             int num_q_heads, int v_dim) {
+    const int64_t t = blockIdx.x;
+    const int h = blockIdx.y, lane = threadIdx.x;
+    const float* mine = part + (t * num_q_heads + h) * shares * (int64_t)(2 + v_dim);
+    float m = -INFINITY;
+    for (int s = 0; s < shares; ++s) m = fmaxf(m, mine[s * (int64_t)(2 + v_dim)]);
+    float l = 0.f;
+    float acc[ATT_ACC];
+#pragma unroll
+    for (int i = 0; i < ATT_ACC; ++i) acc[i] = 0.f;
+    for (int s = 0; s < shares; ++s) {
+        const float* p = mine + s * (int64_t)(2 + v_dim);
+        if (p[0] == -INFINITY) continue;
+        const float f = nva_exp(p[0] - m);
+        l += p[1] * f;
+#pragma unroll
+        for (int i = 0; i < ATT_ACC; ++i) {
+            const int d = lane + i * NVA_WAVE;
+            if (d < v_dim) acc[i] += p[2 + d] * f;
+        }
+    }
+    const float inv = l > 0.f ? 1.f / l : 0.f;
     T* orow = out + t * out_stride + (int64_t)h * v_dim;
 #pragma unroll
     for (int i = 0; i < ATT_ACC; ++i) {
@@ -426,20 +481,27 @@ NVA_EXPORT int NVA_NAME(nva_paged_attention_generic)(
     const void* q, int64_t q_stride, void* out, int64_t out_stride, const void* k_cache, const void* v_cache,
     const int32_t* block_tables, int table_stride, const int32_t* token_seq, const int32_t* positions,
     int64_t tokens, int num_q_heads, int num_kv_heads, int head_dim, int v_dim, int page_size, float scale,
-    int window, int chunk, int keep_first, float softcap, const float* sinks, int32_t* error_flag, hipStream_t stream) {
+    int window, int chunk, int keep_first, float softcap, const float* sinks, float* part, int shares, int32_t* error_flag,
+    hipStream_t stream) {
     if (tokens == 0) return 0;
     if (tokens < 0 || tokens > 0x7fffffff) return nva_fail("paged_attention: bad token count %lld", (long long)tokens);
+    if (shares < 1 || shares > 64 || (shares > 1 && !part))
+        return nva_fail("paged_attention: %d shares of a token's keys (1 to 64, with memory for their results)", shares);
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads || num_q_heads > 65535)
         return nva_fail("paged_attention: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
     if (head_dim <= 0 || head_dim > ATT_MAX_D || v_dim <= 0 || v_dim > ATT_MAX_D)
         return nva_fail("paged_attention: head sizes %d / %d are outside 1..%d", head_dim, v_dim, ATT_MAX_D);
     if (page_size <= 0 || table_stride <= 0) return nva_fail("paged_attention: bad page size or table width");
     if (window < 0 || chunk < 0 || keep_first < 0) return nva_fail("paged_attention: negative window, chunk or kept positions");
-    dim3 grid((unsigned)tokens, (unsigned)num_q_heads);
+    dim3 grid((unsigned)tokens, (unsigned)num_q_heads, (unsigned)shares);
     hipLaunchKernelGGL(paged_attention_generic_kernel<elem_t>, grid, dim3(NVA_WAVE), 0, stream, (const elem_t*)q,
                        q_stride, (elem_t*)out, out_stride, (const elem_t*)k_cache, (const elem_t*)v_cache,
                        block_tables, table_stride, token_seq, positions, num_q_heads, num_kv_heads, head_dim,
-                       v_dim, page_size, scale, window, chunk, keep_first, softcap, sinks, error_flag);
+                       v_dim, page_size, scale, window, chunk, keep_first, softcap, sinks, shares > 1 ? part : nullptr,
+                       error_flag);
+    if (shares > 1)
+        hipLaunchKernelGGL(paged_attention_merge_kernel<elem_t>, dim3((unsigned)tokens, (unsigned)num_q_heads), dim3(NVA_WAVE), 0,
+                           stream, part, shares, (elem_t*)out, out_stride, num_q_heads, v_dim);
     return nva_check_launch("paged_attention_generic");
 }
 

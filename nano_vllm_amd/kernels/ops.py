@@ -301,6 +301,8 @@ class HipKernels:
         self.retention_blocks_side_by_side = True
         # False: the general kernel runs one wave per token for portions of prompts too (the same bits, slower)
         self.tiled_general_attention = True
+        # False: the general kernel walks all of a token's keys in one workgroup, however many
+        self.shared_general_attention = True
         # False: the state-space layer runs a portion's tokens one after the other, whatever its length
         self.state_space_blocks_side_by_side = True
         # how the recurrence holds a state of 65 to 128 rows: 0 two lanes a column (what serves), 1 a thread a column
@@ -1310,12 +1312,18 @@ class HipKernels:
             tokens = batch.num_decode            # what is left: the single tokens before the portions
         if start < tokens:
             n = tokens - start
+            # Few tokens with many keys each: a token's keys are shared out among several workgroups, a share of 128
+            # keys or more, and a second kernel joins their results (a wave alone walks its keys one block after the
+            # other).  The number of shares follows from the step's longest request and the number of tokens alone.
+            reach = min(x for x in (batch.max_kv_len, (window + keep) if window else None, chunk) if x)
+            shares = max(1, min(16, reach // 128, 4096 // (n * num_heads))) if self.shared_general_attention else 1
+            part = torch.empty(n * num_heads * shares * (2 + v_dim), dtype=torch.float32, device=q.device) if shares > 1 else None
             library.call("attn_generic", _suffix(q), "nva_paged_attention_generic", _p(q[start:start + n]), c_i64(qs),
                          _p(out[start:]), c_i64(os_), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
                          _p(batch.token_seq[start:]), _p(batch.positions[start:]), c_i64(n), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(v_dim), c_i32(page_size), c_f32(scale),
-                         c_i32(window or 0), c_i32(chunk or 0), c_i32(keep), c_f32(cap), _p(sinks), _p(self.fault_flag),
-                         self._stream())
+                         c_i32(window or 0), c_i32(chunk or 0), c_i32(keep), c_f32(cap), _p(sinks), _p(part), c_i32(shares),
+                         _p(self.fault_flag), self._stream())
         return out
 
     # ------------------------------------------------------------------ delta rule

@@ -219,7 +219,7 @@ def _attention_case(dtype, dev, hq, hkv, D, DV, page, lens, q_lens, seed, window
         held = set(range(len(mine)))
         if free_passed and window is not None:
             first_needed = max(0, (n - q_lens[s]) - window + 1) // page
-            held = set(range(first_needed, len(mine))) | set(range((keep + page - 1) // page))
+            held = set(range(first_needed, len(mine))) | set(range(min(len(mine), (keep + page - 1) // page)))
         for p in held:
             tables[s, p] = mine[p]
         kk = torch.randn((n, hkv, D), generator=g).to(dtype)
@@ -285,6 +285,21 @@ def test_capped_window_attention_with_kept_first_positions_and_a_sink(backend, d
     k, dev = _kernels(backend, dtype)
     for free_passed in (False, True):
         q, kc, vc, batch, (qs, ks, vs) = _attention_case(dtype, dev, hq, hkv, D, DV, page, lens, q_lens, 5, window, keep,
+                                                         free_passed=free_passed)
+        got = _attend(k, dev, q, hq, hkv, D, DV, kc, vc, batch, 0.3, cap, window, keep)
+        _close(got, _plain_attention(qs, ks, vs, lens, q_lens, 0.3, cap, window, keep), dtype, (window, keep, free_passed))
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq,hkv,D,DV,window,keep,cap", [(4, 2, 16, 24, 600, 37, 4.0), (2, 1, 64, 64, None, 0, None), (8, 2, 128, 128, 300, 130, 30.0)])
+def test_single_tokens_with_many_keys(backend, dtype, hq, hkv, D, DV, window, keep, cap):
+    """Decoded tokens alone in a step, far into their sequences: the kernel shares a token's keys out among several
+    workgroups (the kept positions, the window's blocks, the sink in one share only) and joins the results."""
+    k, dev = _kernels(backend, dtype)
+    lens, q_lens, page = [700, 901, 333, 64, 1], [1, 1, 1, 1, 1], 16
+    for free_passed in (False, True):
+        q, kc, vc, batch, (qs, ks, vs) = _attention_case(dtype, dev, hq, hkv, D, DV, page, lens, q_lens, 11, window, keep,
                                                          free_passed=free_passed)
         got = _attend(k, dev, q, hq, hkv, D, DV, kc, vc, batch, 0.3, cap, window, keep)
         _close(got, _plain_attention(qs, ks, vs, lens, q_lens, 0.3, cap, window, keep), dtype, (window, keep, free_passed))
