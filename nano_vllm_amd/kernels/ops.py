@@ -1316,7 +1316,10 @@ class HipKernels:
             # keys or more, and a second kernel joins their results (a wave alone walks its keys one block after the
             # other).  The number of shares follows from the step's longest request and the number of tokens alone.
             reach = min(x for x in (batch.max_kv_len, (window + keep) if window else None, chunk) if x)
-            shares = max(1, min(16, reach // 128, 4096 // (n * num_heads))) if self.shared_general_attention else 1
+            # (Only where a cap or kept positions keep bfloat16 tokens from the matrix-core decode kernel: everywhere
+            # else this kernel's sums keep the one order that the tiled form for portions shares, bit for bit.)
+            shared = self.shared_general_attention and q.dtype == torch.bfloat16 and (cap > 0.0 or keep > 0)
+            shares = max(1, min(16, reach // 128, 4096 // (n * num_heads))) if shared else 1
             part = torch.empty(n * num_heads * shares * (2 + v_dim), dtype=torch.float32, device=q.device) if shares > 1 else None
             library.call("attn_generic", _suffix(q), "nva_paged_attention_generic", _p(q[start:start + n]), c_i64(qs),
                          _p(out[start:]), c_i64(os_), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),

@@ -292,7 +292,7 @@ def test_capped_window_attention_with_kept_first_positions_and_a_sink(backend, d
 
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hq,hkv,D,DV,window,keep,cap", [(4, 2, 16, 24, 600, 37, 4.0), (2, 1, 64, 64, None, 0, None), (8, 2, 128, 128, 300, 130, 30.0)])
+@pytest.mark.parametrize("hq,hkv,D,DV,window,keep,cap", [(4, 2, 16, 24, 600, 37, 4.0), (2, 1, 64, 64, None, 0, 3.0), (8, 2, 128, 128, 300, 130, 30.0)])
 def test_single_tokens_with_many_keys(backend, dtype, hq, hkv, D, DV, window, keep, cap):
     """Decoded tokens alone in a step, far into their sequences: the kernel shares a token's keys out among several
     workgroups (the kept positions, the window's blocks, the sink in one share only) and joins the results."""
