@@ -17,7 +17,7 @@ from nano_vllm_amd.weights import write_random_model
 
 import plain_kirisun as plain
 
-# Five configurations.  Together: windows smaller and larger than a page and no multiple of it, a window of one
+# Six configurations.  Together: windows smaller and larger than a page and no multiple of it, a window of one
 # position, one longer than every prompt and none at all; 0, 1 and several kept first positions, more of them than
 # a page and more than the window; two windows in one model (two cache groups); 1, 2 and 3 query heads per
 # key/value head; values larger, smaller and as large as keys; rotation of a part of a head, of all of it and none,
@@ -70,6 +70,17 @@ CONFIGS: Dict[str, dict] = {
         KirisunLayer("channel_delta", Delta(heads=2, kv_heads=1, dim=128, vdim=128, conv=4, decay_rank=8, gate_rank=8),
                      Moe(experts=10, top=3, ff=72)))),
         page=64, seed=45),
+    # ones and equal values: a single head, a single expert, as many kept positions as the window holds, a window of
+    # whole pages, multipliers of one, tiny heads
+    "f": dict(cfg=KirisunConfig(vocab=50, width=24, eps=1e-6, residual_mult=1.0, embedding_scale=1.0, layers=(
+        KirisunLayer("channel_delta", Delta(heads=1, kv_heads=1, dim=8, vdim=8, conv=2, decay_rank=2, gate_rank=2),
+                     Moe(experts=1, top=1, ff=8)),
+        KirisunLayer("attention", Att(1, 1, 8, 8, 0.35, softcap=None, window=8, keep_first=8, rot_dims=2, rot_base=10.0),
+                     Moe(experts=2, top=2, ff=8)),
+        KirisunLayer("channel_delta", Delta(heads=2, kv_heads=1, dim=4, vdim=6, conv=4, decay_rank=1, gate_rank=1), None),
+        KirisunLayer("attention", Att(2, 1, 4, 4, 0.5, softcap=1.0, window=64, keep_first=64, rot_dims=4, rot_base=1e3,
+                                      rot_factor=2.0), None))),
+        page=8, seed=46),
 }
 
 _folders: Dict[str, str] = {}

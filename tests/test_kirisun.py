@@ -611,7 +611,7 @@ MODEL_TOL = {"float32": 1e-4, "bfloat16": 6e-2}
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "d", "f"])
 def test_every_cutting_gives_the_plain_logits(backend, name):
     c = K.CONFIGS[name]
     n = 70 if (backend, name) == ("cpu", "b") else 110
@@ -627,7 +627,7 @@ def test_every_cutting_gives_the_plain_logits(backend, name):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name", ["a", "b", "d"])
+@pytest.mark.parametrize("name", ["a", "b", "d", "f"])
 def test_bfloat16_follows_the_plain_logits_under_every_cutting(name):
     c = K.CONFIGS[name]
     n = 130
