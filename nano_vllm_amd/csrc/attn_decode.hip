@@ -91,10 +91,15 @@ __device__ __forceinline__ void load_chunk(int base, bf16x8* ka, bf16x8* kb, bf1
 // plan (int32): [0] number of quotas, [1] number of segments, [2 .. 2 + tokens] where each token's
 // segments begin; from decode_plan_quotas_at on, the first segment of every quota (and the number
 // of segments after the last); from decode_plan_segments_at on, eight ints per segment: token,
-// its request's block table row, its position, 1 if it is the token's only segment; lo, hi, -, -.
+// its request's block table row, its position, 1 if it is the token's only segment; lo, hi, and the range of keys
+// that the token sees in this run of its keys (first, end): a chunk's keys outside it are masked.
 __host__ __device__ inline int64_t decode_plan_quotas_at(int64_t tokens) { return (2 + tokens + 1 + 3) / 4 * 4; }
 __host__ __device__ inline int64_t decode_plan_segments_at(int64_t tokens, int64_t max_segments) {
     return (decode_plan_quotas_at(tokens) + (max_segments - tokens) + 2 + 3) / 4 * 4;     // quotas <= segments - tokens
+}
+// The kept first positions that a token's window has passed: keys 0 .. this - 1 are read beside the window's.
+__host__ __device__ inline int decode_kept_end(int first, int window, int keep_first) {
+    return window > 0 && keep_first > 0 ? (keep_first < first ? keep_first : first) : 0;
 }
 __host__ __device__ inline int decode_quota_cap(int page_size) {
     const int cap = (62 * page_size) / DEC_CHUNK;
@@ -103,8 +108,8 @@ __host__ __device__ inline int decode_quota_cap(int page_size) {
 
 __global__ void __launch_bounds__(NVA_WAVE)
 attn_decode_plan_kernel(const int32_t* __restrict__ positions, const int32_t* __restrict__ token_seq, int tokens,
-                        int page_size, int window, int chunk, int max_segments, int waves_per_head, int32_t* __restrict__ plan,
-                        int32_t* error_flag) {
+                        int page_size, int window, int chunk, int keep_first, int max_segments, int waves_per_head,
+                        int32_t* __restrict__ plan, int32_t* error_flag) {
     const int lane = threadIdx.x;
     // every lane's tokens: position (-1: no such token) and the chunks it sees
     int pos_r[DEC_MAX_TOKENS / NVA_WAVE];
@@ -118,7 +123,7 @@ attn_decode_plan_kernel(const int32_t* __restrict__ positions, const int32_t* __
     for (int i = 0; i < DEC_MAX_TOKENS / NVA_WAVE; ++i)
         if (pos_r[i] >= 0) {
             const int first = nva_first_key(pos_r[i], window, chunk);
-            total += pos_r[i] / DEC_CHUNK - first / DEC_CHUNK + 1;
+            total += pos_r[i] / DEC_CHUNK - first / DEC_CHUNK + 1 + (decode_kept_end(first, window, keep_first) + DEC_CHUNK - 1) / DEC_CHUNK;
         }
 #pragma unroll
     for (int off = NVA_WAVE / 2; off > 0; off >>= 1) total += __shfl_xor(total, off, NVA_WAVE);
@@ -141,7 +146,12 @@ attn_decode_plan_kernel(const int32_t* __restrict__ positions, const int32_t* __
         const int t = i * NVA_WAVE + lane;
         const int pos = pos_r[i];
         const int first = nva_first_key(pos, window, chunk);
-        const int c = pos >= 0 && num_quotas > 0 ? pos / DEC_CHUNK - first / DEC_CHUNK + 1 : 0;
+        const bool planned = pos >= 0 && num_quotas > 0;
+        // the token's chunks, counted through: those of the kept first positions that its window has passed (keys
+        // from 0), then those from its first key on
+        const int kept_end = decode_kept_end(first, window, keep_first);
+        const int ck = planned ? (kept_end + DEC_CHUNK - 1) / DEC_CHUNK : 0;
+        const int c = planned ? ck + pos / DEC_CHUNK - first / DEC_CHUNK + 1 : 0;
         int incl = c;
 #pragma unroll
         for (int off = 1; off < NVA_WAVE; off <<= 1) {
@@ -150,7 +160,9 @@ attn_decode_plan_kernel(const int32_t* __restrict__ positions, const int32_t* __
         }
         const int cum = chunks_before + incl - c;                   // the token's first chunk, counted through
         chunks_before += __shfl(incl, NVA_WAVE - 1, NVA_WAVE);
-        const int n = c > 0 ? (cum + c - 1) / quota - cum / quota + 1 : 0;
+        // each of the two runs is cut by the quotas' edges by itself
+        const int nk = ck > 0 ? (cum + ck - 1) / quota - cum / quota + 1 : 0;
+        const int n = nk + (c > 0 ? (cum + c - 1) / quota - (cum + ck) / quota + 1 : 0);
         incl = n;
 #pragma unroll
         for (int off = 1; off < NVA_WAVE; off <<= 1) {
@@ -163,13 +175,17 @@ attn_decode_plan_kernel(const int32_t* __restrict__ positions, const int32_t* __
             begin[t] = mine;
             const int seq = token_seq[t];
             for (int k = 0; k < n; ++k) {
-                const int qi = cum / quota + k;
-                const int c_lo = max(cum, qi * quota), c_hi = min(cum + c, (qi + 1) * quota);
-                const int lo = (first / DEC_CHUNK + c_lo - cum) * DEC_CHUNK;
-                const int hi = min((first / DEC_CHUNK + c_hi - cum) * DEC_CHUNK, pos + 1);
+                const bool kept = k < nk;
+                const int run_lo = kept ? cum : cum + ck, run_hi = kept ? cum + ck : cum + c;      // the run's chunks
+                const int qi = run_lo / quota + (kept ? k : k - nk);
+                const int c_lo = max(run_lo, qi * quota), c_hi = min(run_hi, (qi + 1) * quota);
+                const int key0 = kept ? 0 : first / DEC_CHUNK * DEC_CHUNK;                         // of the run's first chunk
+                const int seen_lo = kept ? 0 : first, seen_hi = kept ? kept_end : pos + 1;         // the keys seen in this run
+                const int lo = key0 + (c_lo - run_lo) * DEC_CHUNK;
+                const int hi = min(key0 + (c_hi - run_lo) * DEC_CHUNK, seen_hi);
                 if (mine + k < max_segments) {
                     segments[2 * (mine + k)] = make_int4(t, seq, pos, n == 1);
-                    segments[2 * (mine + k) + 1] = make_int4(lo, hi, 0, 0);
+                    segments[2 * (mine + k) + 1] = make_int4(lo, hi, seen_lo, seen_hi);
                     if (c_lo == qi * quota) quota_first[qi] = mine + k;
                 }
             }
@@ -189,7 +205,7 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
                    float* __restrict__ part_o, float* __restrict__ part_ml, const int32_t* __restrict__ plan,
                    const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
                    const int32_t* __restrict__ block_tables, int table_stride, int tokens, int max_segments,
-                   int num_q_heads, int num_kv_heads, int page_size, float scale, int window, int chunk,
+                   int num_q_heads, int num_kv_heads, int page_size, float scale, float softcap,
                    const float* __restrict__ sinks, int32_t* error_flag) {
     constexpr int KP = D / 32;          // 16-byte pieces of a key row per lane = MFMAs per S tile
     constexpr int DT = D / 16;          // 16-channel tiles of the output
@@ -211,7 +227,6 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
 
     // A segment's block table entries: lane i keeps the entry of page lo / page_size + i (a segment
     // spans at most 62 pages, so no chunk needs the table again).
-    auto first_of = [&](const int4& r) { return nva_first_key(r.z, window, chunk); };
     auto window_of = [&](const int4& r, int lo) {
         const int page0 = lo / page_size;
         return page0 + lane <= r.z / page_size ? block_tables[(int64_t)r.y * table_stride + page0 + lane] : -1;
@@ -229,39 +244,38 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
     // load that follows a segment's last chunk is the next segment's first chunk.  (After the
     // quota's last segment the same segment is read once more and dropped.)
     int4 rec = segments[2 * seg];
-    int lo = segments[2 * seg + 1].x, hi = segments[2 * seg + 1].y;
+    const int4 range = segments[2 * seg + 1];
+    int lo = range.x, hi = range.y, first = range.z, kv_len = range.w;       // kv_len: the end of the keys seen in this run
     int table_window = window_of(rec, lo);
     bf16x8 qf[KP];
     load_q(rec, qf);
     bf16x8 ka_n[KP], kb_n[KP], vf_n[DT];
-    load_chunk<D>(lo, ka_n, kb_n, vf_n, k_cache, v_cache, table_window, lo / page_size, first_of(rec), rec.z + 1,
+    load_chunk<D>(lo, ka_n, kb_n, vf_n, k_cache, v_cache, table_window, lo / page_size, first, kv_len,
                   num_kv_heads, kvh, page_size, row_key, col, g, error_flag);
     int seg_next = min(seg + 1, seg_end - 1);
     int4 rec_next = segments[2 * seg_next];
-    int2 range_next = *reinterpret_cast<const int2*>(&segments[2 * seg_next + 1]);
+    int4 range_next = segments[2 * seg_next + 1];
 
     for (;;) {                                                           // over the quota's segments
     const int64_t t = rec.x;
-    const int first = first_of(rec);
-    const int kv_len = rec.z + 1;
     const int window_page0 = lo / page_size;
     // the next segment: its table entries and its query (asked for now, used after this segment)
     // (after the quota's last segment there is none: the loads past its end then all meet the
     // segment's last key, which is visible and whose page the wave's table entries hold)
     const bool more = seg + 1 < seg_end;
     const int lo_next = range_next.x, hi_next = range_next.y;
-    const int first_next = more ? first_of(rec_next) : hi_next - 1;
-    const int kv_len_next = more ? rec_next.z + 1 : hi_next;
+    const int first_next = more ? range_next.z : hi_next - 1;
+    const int kv_len_next = more ? range_next.w : hi_next;
     int table_window_next = table_window;
     bf16x8 qf_next[KP];
     int4 rec_after = rec_next;
-    int2 range_after = range_next;
+    int4 range_after = range_next;
     const int seg_after = min(seg_next + 1, seg_end - 1);
     if (more) {
         table_window_next = window_of(rec_next, lo_next);
         load_q(rec_next, qf_next);
         rec_after = segments[2 * seg_after];
-        range_after = *reinterpret_cast<const int2*>(&segments[2 * seg_after + 1]);
+        range_after = segments[2 * seg_after + 1];
     }
     if (col >= G) {
 #pragma unroll
@@ -275,6 +289,9 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
     for (int i = 0; i < DT; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;      // the maximum in units of raw scores
     const float c_exp = scale * 1.4426950408889634f;      // scale * log2(e)
+    // a cap on the scores, in the raw scores' units: s <- (cap / scale) tanh(s scale / cap), tanh(y) = 1 - 2 / (1 + e^(2 y))
+    const bool capped = softcap > 0.f;
+    const float cap_in = capped ? 2.f * 1.4426950408889634f * scale / softcap : 0.f, cap_out = capped ? softcap / scale : 0.f;
     // The loads of the chunk after are issued, unconditionally and on one path, before the products
     // of the current chunk, so that a wave always has a chunk (16 KiB at head_dim 128) in flight and
     // the wait before the products covers exactly the current chunk's loads.
@@ -319,7 +336,9 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int key = base + 8 * g + i;
-            s[i] = (key >= first && key < kv_len) ? (i < 4 ? sa[i] : sb[i - 4]) : -INFINITY;
+            float raw = i < 4 ? sa[i] : sb[i - 4];
+            if (capped) raw = cap_out - 2.f * cap_out * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(raw * cap_in));
+            s[i] = (key >= first && key < kv_len) ? raw : -INFINITY;
             m_new = fmaxf(m_new, s[i]);
         }
         m_new = nva_max_over_rows(m_new);
@@ -381,6 +400,8 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
     table_window = table_window_next;
     lo = lo_next;
     hi = hi_next;
+    first = first_next;
+    kv_len = kv_len_next;
 #pragma unroll
     for (int c = 0; c < KP; ++c) qf[c] = qf_next[c];
     }
@@ -542,12 +563,15 @@ static int decode_resident_waves(int head_dim) {
 // of the kv heads), and the size of the plan (int32).  Partial results: max_segments * num_q_heads *
 // (head_dim + 2) floats.
 NVA_EXPORT int nva_attn_decode_plan_size_bf16(int longest, int64_t tokens, int num_kv_heads, int head_dim, int page_size,
-                                              int* max_segments, int* waves, int64_t* plan_ints) {
+                                              int keep_first, int* max_segments, int* waves, int64_t* plan_ints) {
     if (longest <= 0 || tokens <= 0 || tokens > DEC_MAX_TOKENS || num_kv_heads <= 0 || page_size <= 0 ||
         !max_segments || !waves || !plan_ints)
         return nva_fail("attn_decode_plan_size: bad arguments (at most %d tokens a launch)", DEC_MAX_TOKENS);
     // a token sees at most longest / 32 + 2 chunks (a window may begin and end inside a chunk)
-    const int64_t chunks = tokens * ((int64_t)longest / DEC_CHUNK + 2);
+    // (and the chunks of its kept first positions, a run of their own with segments of its own)
+    if (keep_first < 0) return nva_fail("attn_decode_plan_size: %d kept positions", keep_first);
+    const int64_t kept_chunks = ((int64_t)keep_first + DEC_CHUNK - 1) / DEC_CHUNK;
+    const int64_t chunks = tokens * ((int64_t)longest / DEC_CHUNK + 2 + kept_chunks);
     const int resident = decode_resident_waves(head_dim);
     if (!resident) return -1;
     int64_t per_head = resident / num_kv_heads > 0 ? resident / num_kv_heads : 1;
@@ -568,7 +592,7 @@ NVA_EXPORT int nva_attn_decode_plan_size_bf16(int longest, int64_t tokens, int n
         per_head -= per_head % (decode_cus / num_kv_heads);
     const int64_t cap = decode_quota_cap(page_size);
     const int64_t quotas = per_head > (chunks + cap - 1) / cap ? per_head : (chunks + cap - 1) / cap;
-    const int64_t bound = tokens + quotas;
+    const int64_t bound = tokens * (keep_first > 0 ? 2 : 1) + quotas;
     if (bound * num_kv_heads > 0x7fffffff || per_head * num_kv_heads > 0x7fffffff)
         return nva_fail("attn_decode_plan_size: too many segments");
     *max_segments = (int)bound;
@@ -580,14 +604,15 @@ NVA_EXPORT int nva_attn_decode_plan_size_bf16(int longest, int64_t tokens, int n
 // Makes the plan of a step (once per step and cache group; every layer's attention reads it).
 // max_segments and waves from nva_attn_decode_plan_size for the same tokens, kv heads and page size.
 NVA_EXPORT int nva_attn_decode_plan_bf16(const int32_t* positions, const int32_t* token_seq, int64_t tokens,
-                                         int num_kv_heads, int page_size, int window, int chunk, int max_segments,
-                                         int waves, int32_t* plan, int32_t* error_flag, hipStream_t stream) {
+                                         int num_kv_heads, int page_size, int window, int chunk, int keep_first,
+                                         int max_segments, int waves, int32_t* plan, int32_t* error_flag,
+                                         hipStream_t stream) {
     if (!positions || !token_seq || !plan || !nva_aligned(plan, 16) || tokens <= 0 || tokens > DEC_MAX_TOKENS ||
-        num_kv_heads <= 0 || page_size <= 0 || window < 0 || chunk < 0 || max_segments <= tokens || waves <= 0 ||
-        waves % num_kv_heads)
+        num_kv_heads <= 0 || page_size <= 0 || window < 0 || chunk < 0 || keep_first < 0 || max_segments <= tokens ||
+        waves <= 0 || waves % num_kv_heads)
         return nva_fail("attn_decode_plan: bad arguments");
     hipLaunchKernelGGL(attn_decode_plan_kernel, dim3(1), dim3(NVA_WAVE), 0, stream, positions, token_seq, (int)tokens,
-                       page_size, window, chunk, max_segments, waves / num_kv_heads, plan, error_flag);
+                       page_size, window, chunk, keep_first, max_segments, waves / num_kv_heads, plan, error_flag);
     return nva_check_launch("attn_decode_plan");
 }
 
@@ -598,7 +623,7 @@ NVA_EXPORT int nva_attn_decode_plan_bf16(const int32_t* positions, const int32_t
 NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride, float* scratch,
                                     const int32_t* plan, const void* k_cache, const void* v_cache,
                                     const int32_t* block_tables, int table_stride, int64_t tokens, int num_q_heads,
-                                    int num_kv_heads, int head_dim, int page_size, float scale, int window, int chunk,
+                                    int num_kv_heads, int head_dim, int page_size, float scale, float softcap,
                                     int max_segments, int waves, const float* sinks, int32_t* error_flag,
                                     hipStream_t stream) {
     if (tokens == 0) return 0;
@@ -618,17 +643,17 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
     if (tokens < 0 || tokens > DEC_MAX_TOKENS || num_q_heads > 65535)
         return nva_fail("attn_decode: %lld tokens (at most %d a launch) or %d heads exceed the grid", (long long)tokens,
                         DEC_MAX_TOKENS, num_q_heads);
-    if (max_segments <= tokens || waves <= 0 || waves % num_kv_heads || window < 0 || chunk < 0 || table_stride <= 0 || !scratch ||
-        !plan || !nva_aligned(plan, 16))
-        return nva_fail("attn_decode: bad plan (%d segments, %d waves), window %d or no scratch", max_segments, waves,
-                        window);
+    if (max_segments <= tokens || waves <= 0 || waves % num_kv_heads || !(softcap >= 0.f) || !(softcap <= 3.0e38f) ||
+        table_stride <= 0 || !scratch || !plan || !nva_aligned(plan, 16))
+        return nva_fail("attn_decode: bad plan (%d segments, %d waves), cap %g or no scratch", max_segments, waves,
+                        (double)softcap);
     float* part_o = scratch;
     float* part_ml = scratch + (int64_t)max_segments * num_q_heads * head_dim;
 #define LAUNCH(DD)                                                                                              \
     hipLaunchKernelGGL(attn_decode_kernel<DD>, dim3((unsigned)waves), dim3(NVA_WAVE), 0, stream, (const __bf16*)q, \
                        q_stride, (__bf16*)out, out_stride, part_o, part_ml, plan, (const __bf16*)k_cache,         \
                        (const __bf16*)v_cache, block_tables, table_stride, (int)tokens, max_segments, num_q_heads,  \
-                       num_kv_heads, page_size, scale, window, chunk, sinks, error_flag)
+                       num_kv_heads, page_size, scale, softcap, sinks, error_flag)
     switch (head_dim) {
         case 32: LAUNCH(32); break;
         case 64: LAUNCH(64); break;

@@ -1282,13 +1282,11 @@ class HipKernels:
         if cap < 0.0 or keep < 0:
             raise KernelError("attention: a negative softcap or number of kept positions")
         mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and v_dim == head_dim
-        # (the decode kernel knows neither a cap on the scores nor kept first positions: such single tokens run the
-        # general kernel, the portions of prompts beside them the matrix-core prefill kernel all the same)
-        if batch.num_decode > 0 and mfma and cap == 0.0 and keep == 0 and \
+        if batch.num_decode > 0 and mfma and \
                 self._decode_kernel_takes(num_heads // num_kv_heads, head_dim, page_size, q, qs, out, os_):
             start = batch.num_decode
             self._attention_decode(q, qs, out, os_, k_cache, v_cache, tables, batch, start, num_heads, num_kv_heads,
-                                   head_dim, page_size, scale, window, sinks, chunk)
+                                   head_dim, page_size, scale, window, sinks, chunk, keep, cap)
         if batch.num_decode < tokens and mfma and \
                 self._prefill_kernel_takes(head_dim, page_size, tables.shape[1], q, qs, out, os_):
             # portions of prompts: the matrix-core prefill kernel, one workgroup per 32 query rows
@@ -1590,7 +1588,7 @@ class HipKernels:
                                                                              out_stride)
 
     def _attention_decode(self, q, qs, out, os_, k_cache, v_cache, tables, batch, n, num_heads, num_kv_heads,
-                          head_dim, page_size, scale, window, sinks=None, chunk=None):
+                          head_dim, page_size, scale, window, sinks=None, chunk=None, keep=0, cap=0.0):
         # The work is shared out on the device from the tokens' positions, once per step and (kv
         # heads, window): the first layer that asks makes the plan, the others find it on the batch.
         # The library says how large the partial results may get for this many tokens of at most
@@ -1600,25 +1598,25 @@ class HipKernels:
             plans = batch.step_cache = {}
         for t0 in range(0, n, 1024):
             t1 = min(n, t0 + 1024)
-            key = ("decode_plan", t0, num_kv_heads, head_dim, page_size, window or 0, chunk or 0)
+            key = ("decode_plan", t0, num_kv_heads, head_dim, page_size, window or 0, chunk or 0, keep)
             if key not in plans:
                 bound, waves, ints = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int64(0)
                 library.call("attn_decode", "bf16", "nva_attn_decode_plan_size", c_i32(batch.max_kv_len), c_i64(t1 - t0),
-                             c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), ctypes.byref(bound),
+                             c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_i32(keep), ctypes.byref(bound),
                              ctypes.byref(waves), ctypes.byref(ints))
                 plan = torch.empty(ints.value, dtype=torch.int32, device=q.device)
                 library.call("attn_decode", "bf16", "nva_attn_decode_plan", _p(batch.positions[t0:t1]),
                              _p(batch.token_seq[t0:t1]), c_i64(t1 - t0),
-                             c_i32(num_kv_heads), c_i32(page_size), c_i32(window or 0), c_i32(chunk or 0), c_i32(bound.value),
-                             c_i32(waves.value), _p(plan), _p(self.fault_flag), self._stream())
+                             c_i32(num_kv_heads), c_i32(page_size), c_i32(window or 0), c_i32(chunk or 0), c_i32(keep),
+                             c_i32(bound.value), c_i32(waves.value), _p(plan), _p(self.fault_flag), self._stream())
                 plans[key] = (plan, bound.value, waves.value)
             plan, bound, waves = plans[key]
             scratch = torch.empty(bound * num_heads * (head_dim + 2), dtype=torch.float32, device=q.device)
             library.call("attn_decode", "bf16", "nva_attn_decode", _p(q[t0:t1]), c_i64(qs), _p(out[t0:t1]), c_i64(os_),
                          _p(scratch), _p(plan), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
                          c_i64(t1 - t0), c_i32(num_heads),
-                         c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
-                         c_i32(chunk or 0), c_i32(bound), c_i32(waves), _p(sinks), _p(self.fault_flag), self._stream())
+                         c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_f32(cap),
+                         c_i32(bound), c_i32(waves), _p(sinks), _p(self.fault_flag), self._stream())
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:

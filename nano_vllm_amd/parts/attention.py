@@ -126,8 +126,6 @@ class Attention(Part):
         rope = ("rope",) if self.row_prepare and self.position_encoding else ()
         if self.v_head_dim != self.head_dim:
             return (prepare, "attn_generic") + rope
-        if self.softcap is not None or self.keep_first:        # single tokens run the general kernel
-            return (prepare, "attn_generic", "attn_prefill") + rope
         return (prepare, "attn_generic", "attn_decode", "attn_prefill") + \
             (("rope",) if self.row_prepare and self.position_encoding else ())
 
