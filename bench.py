@@ -94,7 +94,7 @@ def mafarax_config(width: int, layers: int, dtype: str) -> dict:
 def kirisun_config(width: int, layers: int, dtype: str) -> dict:
     """A Kirisun model of the width's layer sizes: delta-rule layers with as many value heads of 128 channels as
     the dense model has query heads (a state of 128 x 128 a head) and attention layers with the dense model's heads
-    (a window of 1024 positions that keeps the first 4, scores capped at 50, half the head rotated) in turn; 32
+    (a window of 1024 positions that keeps the first 4, scores capped at 30, half the head rotated) in turn; 32
     gated experts of an eighth of the dense inner size of which a token runs 8."""
     from nano_vllm_amd.models.shapes import _kirisun
     heads, kv, dim, inner = DESIGN_SIZES[width]

@@ -58,7 +58,7 @@ def _mafarax(layers, width, heads, kv_heads, dim, vdim, inner, vocab, chunk, eps
 
 
 def _kirisun(layers, width, heads, kv_heads, dim, vdim, inner, vocab, window, keep_first=4, eps=1e-6, dtype="bfloat16",
-             rot=None, factor=2.0, softcap=50.0, delta_heads=None, delta_kv_heads=None, delta_dim=None, delta_vdim=None, conv=4,
+             rot=None, factor=4.0, softcap=30.0, delta_heads=None, delta_kv_heads=None, delta_dim=None, delta_vdim=None, conv=4,
              rank=None, experts=32, top=8, residual_mult=0.5, pattern=("channel_delta", "attention")) -> dict:
     """Layers that follow `pattern` in turn: the gated window attention (a cap on the scores, kept first positions,
     half the head rotated) and the channel-wise delta rule (as many value heads of the same size as the attention's
@@ -76,7 +76,7 @@ def _kirisun(layers, width, heads, kv_heads, dim, vdim, inner, vocab, window, ke
                                     "decay_rank": rank or max(1, dd // 2), "gate_rank": rank or max(1, dd // 2)}},
     }
     return {"architecture": "Kirisun", "vocab": vocab, "width": width, "norm": {"eps": eps}, "residual_mult": residual_mult,
-            "embedding": {"scale": float(width) ** 0.5}, "layers": [kinds[pattern[i % len(pattern)]] for i in range(layers)],
+            "embedding": {"scale": 8.0}, "layers": [kinds[pattern[i % len(pattern)]] for i in range(layers)],
             "torch_dtype": dtype}
 
 

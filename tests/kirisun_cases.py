@@ -62,7 +62,7 @@ CONFIGS: Dict[str, dict] = {
         page=16, seed=44),
     # a larger one for long prompts: heads of 64 to 128, windows over several pages, a delta-rule head wider than a wave
     "e": dict(cfg=KirisunConfig(vocab=384, width=256, eps=1e-5, residual_mult=0.4, embedding_scale=16.0, layers=(
-        KirisunLayer("attention", Att(4, 2, 64, 64, 0.125, softcap=40.0, window=160, keep_first=70, rot_dims=64, rot_base=2e4,
+        KirisunLayer("attention", Att(4, 2, 64, 64, 0.11, softcap=40.0, window=160, keep_first=70, rot_dims=64, rot_base=2e4,
                                       rot_factor=1.0), Moe(experts=10, top=3, ff=72)),
         KirisunLayer("channel_delta", Delta(heads=4, kv_heads=4, dim=96, vdim=80, conv=3, decay_rank=8, gate_rank=8), None),
         KirisunLayer("attention", Att(2, 1, 128, 128, 0.09, softcap=40.0, window=70, keep_first=1, rot_dims=32, rot_base=2e4,

@@ -112,7 +112,7 @@ def test_the_scaled_embedding_starts_a_float_stream(backend, dtype):
 
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width,mult", [(48, 0.5), (20, 1.0), (320, 0.3), (1000, 2.0)])
+@pytest.mark.parametrize("width,mult", [(48, 0.5), (20, 1.0), (328, 0.35), (1000, 2.0)])
 def test_a_normed_addend_goes_into_the_float_stream(backend, dtype, width, mult):
     """r <- r + mult * n_a(a), y = n(r): the stream stays float32 (far beyond bfloat16's grain), y is rounded once."""
     k, dev = _kernels(backend, dtype)
@@ -276,7 +276,7 @@ def _attend(k, dev, q, hq, hkv, D, DV, kc, vc, batch, scale, cap, window, keep):
     (2, 1, 64, 64, 32, 48, 4, 30.0, [97, 150], [1, 85]),                         # sizes of the matrix-core kind
     (2, 2, 8, 8, 4, 4096, 5, None, [70, 130], [1, 130]),                         # a window longer than every request, no cap
     (2, 1, 10, 10, 4, None, 0, 1.5, [50, 21], [1, 21]),                          # no window at all
-    (4, 1, 64, 64, 16, 40, 0, 50.0, [120, 90], [1, 60]),                         # a window without kept positions
+    (4, 2, 64, 64, 16, 56, 0, 25.0, [120, 90], [1, 60]),                         # a window without kept positions
     (8, 2, 128, 128, 64, 96, 70, 20.0, [500, 260], [1, 260])])
 def test_capped_window_attention_with_kept_first_positions_and_a_sink(backend, dtype, hq, hkv, D, DV, page, window, keep, cap,
                                                                       lens, q_lens):
@@ -332,9 +332,9 @@ def test_a_key_just_inside_and_just_outside_the_window_and_the_kept_positions(ba
     position and the one after it, hundreds of positions back among the kept; in a prompt's portion and by a
     decoded token, on tables whose passed pages went back."""
     k, dev = _kernels(backend, dtype)
-    window, keep, page = 40, 6, 16
+    window, keep, page = 44, 5, 16
     for q_len in (1, 25):
-        for n in (300, 337, 47, 41, 40):
+        for n in (300, 337, 51, 45, 44):
             last = n - 1
             cases = [(last, True), (last - window + 1, True), (last - window, last - window < keep), (keep - 1, True),
                      (keep, last - keep < window), (0, True), (last - window - 100, False)]
@@ -363,7 +363,7 @@ def test_the_sigmoid_gate(backend, dtype):
 
 # ------------------------------------------------------------------------------ experts
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("experts,top", [(6, 2), (4, 1), (5, 3), (3, 3), (12, 3), (64, 6), (15, 2)])
+@pytest.mark.parametrize("experts,top", [(6, 2), (4, 1), (5, 3), (3, 3), (11, 3), (64, 6), (15, 2)])
 def test_the_largest_logits_are_chosen_and_weighted_among_themselves(backend, experts, top):
     k, dev = _kernels(backend)
     g = torch.Generator().manual_seed(experts * 10 + top)
@@ -417,7 +417,7 @@ def test_the_gated_experts_products(backend, dtype, tokens, width, ff, experts, 
 
 
 # ------------------------------------------------------------------------------ the delta rule
-DELTA_SHAPES = [(4, 2, 12, 8, 3), (2, 2, 10, 14, 1), (3, 1, 5, 7, 5), (2, 1, 40, 70, 2), (4, 4, 64, 64, 4), (2, 1, 128, 128, 4),
+DELTA_SHAPES = [(4, 2, 12, 8, 3), (2, 2, 10, 14, 1), (3, 1, 5, 7, 5), (2, 1, 40, 70, 2), (2, 2, 64, 64, 4), (2, 1, 128, 128, 4),
                 (1, 1, 130, 20, 2)]          # heads, kv_heads, dim, vdim, taps
 
 
