@@ -277,6 +277,8 @@ def _attend(k, dev, q, hq, hkv, D, DV, kc, vc, batch, scale, cap, window, keep):
     (2, 2, 8, 8, 4, 4096, 5, None, [70, 130], [1, 130]),                         # a window longer than every request, no cap
     (2, 1, 10, 10, 4, None, 0, 1.5, [50, 21], [1, 21]),                          # no window at all
     (4, 2, 64, 64, 16, 56, 0, 25.0, [120, 90], [1, 60]),                         # a window without kept positions
+    (2, 1, 64, 64, 16, None, 0, 12.0, [150, 90], [1, 90]),                       # a cap alone, at the matrix cores' sizes
+    (4, 2, 64, 64, 32, 70, 9, None, [200, 131], [1, 131]),                       # kept positions alone
     (8, 2, 128, 128, 64, 96, 70, 20.0, [500, 260], [1, 260])])
 def test_capped_window_attention_with_kept_first_positions_and_a_sink(backend, dtype, hq, hkv, D, DV, page, window, keep, cap,
                                                                       lens, q_lens):
