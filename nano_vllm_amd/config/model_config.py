@@ -687,3 +687,198 @@ class KirisunConfig:
         if self.eos_token_id is not None:
             out["eos_token_id"] = list(self.eos_token_id)
         return out
+
+
+# ---------------------------------------------------------------------------- Pemuvik
+@dataclass(frozen=True)
+class SigmoidAttentionConfig:
+    """Grouped attention without a softmax: a visible key weighs sigmoid(scale q.k + a learned number per head).
+    Biases on all four projections; the first rot_dims channels of every q and k head rotated in neighbouring
+    pairs (0: none); every value head divided by its root mean square; window None: every earlier position;
+    v_mix: the layer mixes its values with those of the model's first such layer."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: Optional[int] = None
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    v_mix: bool = False
+
+
+@dataclass(frozen=True)
+class LatentAttentionConfig:
+    """Causal softmax attention whose keys and values are made from a latent row of kv_rank entries per token and
+    one rotated key part of rot_dim entries shared by the heads; a head's query has dim plain and rot_dim rotated
+    entries; a learned sink per head."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    kv_rank: int
+    scale: float
+    rot_base: float = 10000.0
+
+
+@dataclass(frozen=True)
+class ChoiceExpertsConfig:
+    """A routed feed-forward: `top` of experts + identity router outputs (the last `identity` of them give the input
+    back) in group_count groups of which group_keep can be chosen from; gated experts of inner size ff; shared_ff:
+    the inner size of a shared expert behind a sigmoid gate, or None."""
+    experts: int
+    top: int
+    ff: int
+    identity: int = 0
+    group_count: int = 1
+    group_keep: int = 1
+    shared_ff: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class PemuvikLayer:
+    kind: str                                    # "attention" | "latent_attention"
+    mixer: Any                                   # SigmoidAttentionConfig | LatentAttentionConfig
+    mlp: Any                                     # None | int (a dense layer's inner size) | ChoiceExpertsConfig
+
+
+@dataclass(frozen=True)
+class PemuvikConfig:
+    """Pemuvik: layers whose mixer and feed-forward read a norm each of the same float32 residual stream and are
+    added to it through a learned vector each; the mixer is, layer by layer, a window attention with sigmoid
+    weights or an attention through a shared latent; the feed-forward a dense gated layer, a mixture of gated
+    experts, or absent; the head is the embedding table.  config.json gives every size and constant, layer by layer."""
+    vocab: int
+    width: int
+    eps: float
+    layers: Tuple[PemuvikLayer, ...]
+    dtype: str = "bfloat16"
+    eos_token_id: Optional[Tuple[int, ...]] = None
+    architecture: str = "Pemuvik"
+
+    @classmethod
+    def from_dict(cls, d: Mapping[str, Any]) -> "PemuvikConfig":
+        where = "config.json"
+        entries = d.get("layers")
+        if not isinstance(entries, (list, tuple)) or not entries:
+            raise ConfigError(f"{where}: key 'layers' must be a list of layers")
+        layers = []
+        for i, entry in enumerate(entries):
+            at = f"{where}: layers[{i}]"
+            if not isinstance(entry, Mapping):
+                raise ConfigError(f"{at} must be an object")
+            kind = entry.get("type")
+            m = _section(entry, "mixer", at)
+            ma = at + ".mixer"
+            rot = m.get("rot")
+            dims, base = 0, 10000.0
+            if rot is not None:
+                dims = _whole(rot, "dims", ma + ".rot")
+                base = _require(rot, "base", float, ma + ".rot")
+            if kind == "attention":
+                mask = m.get("mask")
+                mixer = SigmoidAttentionConfig(
+                    heads=_whole(m, "heads", ma), kv_heads=_whole(m, "kv_heads", ma), dim=_whole(m, "dim", ma),
+                    vdim=_whole(m, "vdim", ma), scale=_require(m, "scale", float, ma),
+                    window=None if mask is None else _whole(mask, "size", ma + ".mask"),
+                    rot_dims=dims, rot_base=base, v_mix=bool(m.get("v_mix", False)))
+            elif kind == "latent_attention":
+                mixer = LatentAttentionConfig(
+                    heads=_whole(m, "heads", ma), dim=_whole(m, "dim", ma), rot_dim=_whole(m, "rot_dim", ma),
+                    vdim=_whole(m, "vdim", ma), kv_rank=_whole(m, "kv_rank", ma), scale=_require(m, "scale", float, ma),
+                    rot_base=base)
+                if rot is None or dims != mixer.rot_dim:
+                    raise ConfigError(f"{ma}: rot.dims must be there and equal rot_dim {mixer.rot_dim}, got {dims}")
+            else:
+                raise ConfigError(f"{at}: type must be 'attention' or 'latent_attention', got {kind!r}")
+            mlp = entry.get("mlp")
+            ff: Any = None
+            if mlp is not None:
+                fa = at + ".mlp"
+                if not isinstance(mlp, Mapping) or mlp.get("kind") not in ("dense", "moe"):
+                    raise ConfigError(f"{fa} must be null or an object of kind 'dense' or 'moe', got {mlp!r}")
+                if mlp["kind"] == "dense":
+                    ff = _whole(mlp, "ff", fa)
+                else:
+                    router = _section(mlp, "router", fa)
+                    groups = router.get("groups") or {}
+                    shared = mlp.get("shared")
+                    ff = ChoiceExpertsConfig(
+                        experts=_whole(router, "experts", fa + ".router"), top=_whole(router, "top", fa + ".router"),
+                        ff=_whole(_section(mlp, "expert", fa), "ff", fa + ".expert"),
+                        identity=_count(router, "identity", fa + ".router", 0),
+                        group_count=_whole(groups, "count", fa + ".router.groups", 1),
+                        group_keep=_whole(groups, "keep", fa + ".router.groups", 1) if groups else 1,
+                        shared_ff=None if shared is None else _whole(shared, "ff", fa + ".shared"))
+            layers.append(PemuvikLayer(kind, mixer, ff))
+        norm = _section(d, "norm", where)
+        eos = d.get("eos_token_id")
+        eos = (eos,) if isinstance(eos, int) else tuple(int(x) for x in eos) if isinstance(eos, (list, tuple)) else None
+        cfg = cls(vocab=_whole(d, "vocab", where), width=_whole(d, "width", where),
+                  eps=_require(norm, "eps", float, where + ": norm"), layers=tuple(layers),
+                  dtype=canonical_dtype(d.get("dtype") or d.get("torch_dtype") or "bfloat16"),
+                  eos_token_id=eos, architecture=d.get("architecture") or (d.get("architectures") or ["Pemuvik"])[0])
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if not (self.eps > 0):
+            raise ConfigError(f"config.json: norm.eps must be positive, got {self.eps}")
+        mixed = None
+        for i, layer in enumerate(self.layers):
+            at = f"config.json: layers[{i}]"
+            m, f = layer.mixer, layer.mlp
+            if not (m.scale > 0):
+                raise ConfigError(f"{at}: scale must be positive, got {m.scale}")
+            if not (m.rot_base > 0):
+                raise ConfigError(f"{at}: rot.base must be positive, got {m.rot_base}")
+            if layer.kind == "attention":
+                if m.heads % m.kv_heads:
+                    raise ConfigError(f"{at}: {m.heads} heads do not divide into {m.kv_heads} kv_heads")
+                if m.rot_dims % 2 or m.rot_dims > m.dim:
+                    raise ConfigError(f"{at}: rot.dims {m.rot_dims} must be even and at most dim {m.dim}")
+                if m.v_mix:
+                    if mixed is not None and mixed != (m.kv_heads, m.vdim):
+                        raise ConfigError(f"{at}: layers that mix values have the same kv_heads and vdim, got "
+                                          f"{(m.kv_heads, m.vdim)} after {mixed}")
+                    mixed = (m.kv_heads, m.vdim)
+            elif m.rot_dim % 2:
+                raise ConfigError(f"{at}: rot_dim {m.rot_dim} must be even")
+            if isinstance(f, ChoiceExpertsConfig):
+                routed = f.experts + f.identity
+                if routed % f.group_count or not 1 <= f.group_keep <= f.group_count:
+                    raise ConfigError(f"{at}: {routed} router outputs in {f.group_count} groups of which {f.group_keep} are kept")
+                if not 1 <= f.top <= f.group_keep * (routed // f.group_count):
+                    raise ConfigError(f"{at}: {f.top} experts a token out of {f.group_keep} groups of {routed // f.group_count}")
+
+    def to_dict(self) -> dict:
+        """The config.json that describes this configuration."""
+        entries = []
+        for layer in self.layers:
+            m, f = layer.mixer, layer.mlp
+            if layer.kind == "attention":
+                mixer = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim, "vdim": m.vdim, "scale": m.scale,
+                         "v_mix": m.v_mix}
+                if m.window is not None:
+                    mixer["mask"] = {"size": m.window}
+                if m.rot_dims:
+                    mixer["rot"] = {"dims": m.rot_dims, "base": m.rot_base}
+            else:
+                mixer = {"heads": m.heads, "dim": m.dim, "rot_dim": m.rot_dim, "vdim": m.vdim, "kv_rank": m.kv_rank,
+                         "scale": m.scale, "rot": {"dims": m.rot_dim, "base": m.rot_base}}
+            if f is None:
+                mlp = None
+            elif isinstance(f, int):
+                mlp = {"kind": "dense", "ff": f}
+            else:
+                mlp = {"kind": "moe", "expert": {"ff": f.ff},
+                       "router": {"experts": f.experts, "top": f.top, "identity": f.identity,
+                                  "groups": {"count": f.group_count, "keep": f.group_keep}}}
+                if f.shared_ff is not None:
+                    mlp["shared"] = {"ff": f.shared_ff}
+            entries.append({"type": layer.kind, "mixer": mixer, "mlp": mlp})
+        out = {"architecture": self.architecture, "vocab": self.vocab, "width": self.width, "norm": {"eps": self.eps},
+               "layers": entries, "torch_dtype": self.dtype}
+        if self.eos_token_id is not None:
+            out["eos_token_id"] = list(self.eos_token_id)
+        return out

@@ -18,6 +18,8 @@
 // softcap > 0: s_j <- softcap * tanh(s_j / softcap) after the scale.  keep_first > 0 (with a window): the keys
 // at positions < keep_first stay visible to every query, however far back; the per-token kernel walks them
 // first, then the window.
+// sig_bias, float [Hq] or null (the per-token kernel): no softmax; a visible key weighs sigmoid(s_j + sig_bias_h) and the
+// weights are not normalised over the keys: o = sum_j sigmoid(s_j + b_h) v_j.  (No sink, no sharing of a token's keys.)
 //
 // Portions of prompts have a second kernel with the same arithmetic, operation for operation (the
 // results are the same bits): a workgroup takes 32 query rows of one request and one head, and the
@@ -38,7 +40,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
                                const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
                                int num_q_heads, int num_kv_heads, int head_dim, int v_dim, int page_size, float scale,
                                int window, int chunk, int keep_first, float softcap, const float* __restrict__ sinks,
-                               float* __restrict__ part, int32_t* error_flag) {
+                               const float* __restrict__ sig_bias, float* __restrict__ part, int32_t* error_flag) {
     __shared__ float q_s[ATT_MAX_D];
     __shared__ float p_s[NVA_WAVE];
     __shared__ int64_t v_off_s[NVA_WAVE];
@@ -67,6 +69,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
     float m_run = with_sink ? sinks[h] : -INFINITY, l_run = with_sink ? 1.f : 0.f;
     const bool vec = head_dim % 8 == 0;
     const int vt = nva_v_tile(page_size);
+    const float sig_b = sig_bias ? sig_bias[h] : 0.f;
 
     // the kept first positions that the window has passed, [0, kept_end), then the window (or chunk) up to pos
     const int kept_end = window > 0 && keep_first > 0 ? min(keep_first, first) : 0;
@@ -116,13 +119,20 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
                 if (softcap > 0.f) s = softcap * tanhf(s / softcap);
             }
         }
+        float p, correction;
+        if (sig_bias) {
+            // every key by itself: no maximum, no sum, nothing to rescale
+            p = (s == -INFINITY) ? 0.f : 1.f / (1.f + nva_exp(-(s + sig_b)));
+            correction = 1.f;
+        } else {
         const float m_new = fmaxf(m_run, wave_max(s));
         // m_new is finite: the key at `pos` itself is always visible in the first chunk that holds it;
         // a chunk of only faulty keys leaves m_new at -inf, guarded below.
-        const float p = (s == -INFINITY) ? 0.f : nva_exp(s - m_new);
-        const float correction = (m_run == -INFINITY) ? 0.f : nva_exp(m_run - m_new);
+        p = (s == -INFINITY) ? 0.f : nva_exp(s - m_new);
+        correction = (m_run == -INFINITY) ? 0.f : nva_exp(m_run - m_new);
         l_run = l_run * correction + wave_sum(p);
         m_run = m_new;
+        }
         __syncthreads();
         p_s[lane] = p;
         v_off_s[lane] = v_off;
@@ -165,7 +175,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
         }
         return;
     }
-    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+    const float inv = sig_bias ? 1.f : l_run > 0.f ? 1.f / l_run : 0.f;
     T* orow = out + t * out_stride + (int64_t)h * v_dim;
 #pragma unroll
     for (int i = 0; i < ATT_ACC; ++i) {
@@ -481,8 +491,8 @@ NVA_EXPORT int NVA_NAME(nva_paged_attention_generic)(
     const void* q, int64_t q_stride, void* out, int64_t out_stride, const void* k_cache, const void* v_cache,
     const int32_t* block_tables, int table_stride, const int32_t* token_seq, const int32_t* positions,
     int64_t tokens, int num_q_heads, int num_kv_heads, int head_dim, int v_dim, int page_size, float scale,
-    int window, int chunk, int keep_first, float softcap, const float* sinks, float* part, int shares, int32_t* error_flag,
-    hipStream_t stream) {
+    int window, int chunk, int keep_first, float softcap, const float* sinks, const float* sig_bias, float* part, int shares,
+    int32_t* error_flag, hipStream_t stream) {
     if (tokens == 0) return 0;
     if (tokens < 0 || tokens > 0x7fffffff) return nva_fail("paged_attention: bad token count %lld", (long long)tokens);
     if (shares < 1 || shares > 64 || (shares > 1 && !part))
@@ -493,12 +503,13 @@ NVA_EXPORT int NVA_NAME(nva_paged_attention_generic)(
         return nva_fail("paged_attention: head sizes %d / %d are outside 1..%d", head_dim, v_dim, ATT_MAX_D);
     if (page_size <= 0 || table_stride <= 0) return nva_fail("paged_attention: bad page size or table width");
     if (window < 0 || chunk < 0 || keep_first < 0) return nva_fail("paged_attention: negative window, chunk or kept positions");
+    if (sig_bias && (sinks || shares > 1)) return nva_fail("paged_attention: sigmoid weights go without a sink and without shares");
     dim3 grid((unsigned)tokens, (unsigned)num_q_heads, (unsigned)shares);
     hipLaunchKernelGGL(paged_attention_generic_kernel<elem_t>, grid, dim3(NVA_WAVE), 0, stream, (const elem_t*)q,
                        q_stride, (elem_t*)out, out_stride, (const elem_t*)k_cache, (const elem_t*)v_cache,
                        block_tables, table_stride, token_seq, positions, num_q_heads, num_kv_heads, head_dim,
-                       v_dim, page_size, scale, window, chunk, keep_first, softcap, sinks, shares > 1 ? part : nullptr,
-                       error_flag);
+                       v_dim, page_size, scale, window, chunk, keep_first, softcap, sinks, sig_bias,
+                       shares > 1 ? part : nullptr, error_flag);
     if (shares > 1)
         hipLaunchKernelGGL(paged_attention_merge_kernel<elem_t>, dim3((unsigned)tokens, (unsigned)num_q_heads), dim3(NVA_WAVE), 0,
                            stream, part, shares, (elem_t*)out, out_stride, num_q_heads, v_dim);

@@ -9,13 +9,20 @@
 //             ids [tokens, top], weights [tokens, top] = scale * s.
 //             With softmax_top the logits (plus an optional float bias per expert) are compared as they are: the
 //             `top` largest are chosen (no groups) and weighted by the softmax over the chosen logits alone.
+//             With softmax_choice (mode 2) s = softmax(z) over all experts; an expert is chosen by s + bias (a float per
+//             expert), a group counts by the largest such choice score in it, only the kept groups' experts can be
+//             chosen (the others do not take part, whatever the sign of the scores); the weights are the chosen
+//             experts' s (without the bias) divided by their sum + 1e-20.
+//             Experts numbered from `experts` on (the kernels of the products are told how many real ones there are)
+//             are identities: their output is the token's input itself.
 //   plan      the pairs (token, choice) counted and sorted by expert: place[pair] = the pair's row among the
 //             sorted ones, rows[place] = pair; the sorted rows cut into tiles of 32 or 128 rows of one expert:
 //             tile_expert[i], tile_row0[i], tile_rows[i], and their number.
 //   up        h[row] = act(x[token of row] Wu_e^T)         rows sorted by expert, a tile of rows and 64 or 128
 //             gated: h[row] = act(x Wg_e^T) * (x Wu_e^T), an expert's matrix holding its gate rows, then its up rows
 //   down      o[row] = h[row] Wd_e^T                       outputs to a workgroup
-//   combine   y[token] = sum over its choices of weight * o[place] (+ add[token])
+//   combine   y[token] = sum over its choices of weight * o[place] (x[token] for an identity) (+ add[token], times
+//             sigmoid(add_gate[token]) where a float gate logit per token is given)
 //
 // The products are float sums of a row by itself (on the vector units over k in ascending order, one chain per
 // output; on the matrix cores in the order of the instruction's steps), so a token's result does not depend on
@@ -44,12 +51,31 @@ __global__ void __launch_bounds__(NVA_WAVE)
 moe_route_kernel(const float* __restrict__ logits, int64_t stride, int experts, int top, int group_count, int group_keep,
                  float scale, int softmax_top, const float* __restrict__ bias, int32_t* __restrict__ ids,
                  float* __restrict__ weights) {
-    __shared__ float s_s[MOE_MAX_EXPERTS];
+    __shared__ float s_s[MOE_MAX_EXPERTS];           // what the experts are compared by
+    __shared__ float w_s[MOE_MAX_EXPERTS];           // softmax_choice: the scores without the bias
     __shared__ float g_s[MOE_MAX_EXPERTS];           // group scores; -inf once taken
     __shared__ unsigned char open_s[MOE_MAX_EXPERTS];
     const int64_t t = blockIdx.x;
     const int lane = threadIdx.x;
     const bool all_groups = group_keep == group_count;
+    const bool choice = softmax_top == 2;
+    if (choice) {
+        float m = -INFINITY;
+        for (int e = lane; e < experts; e += NVA_WAVE) m = fmaxf(m, logits[t * stride + e]);
+        m = wave_max(m);
+        float sum = 0.f;
+        for (int e = lane; e < experts; e += NVA_WAVE) {
+            const float x = expf(logits[t * stride + e] - m);
+            w_s[e] = x;
+            sum += x;
+        }
+        sum = wave_sum(sum);
+        for (int e = lane; e < experts; e += NVA_WAVE) {
+            w_s[e] /= sum;
+            s_s[e] = w_s[e] + (bias ? bias[e] : 0.f);
+            open_s[e] = all_groups ? 1 : 0;
+        }
+    } else
     for (int e = lane; e < experts; e += NVA_WAVE) {
         const float z = logits[t * stride + e] + (bias ? bias[e] : 0.f);
         s_s[e] = softmax_top ? z : 1.f / (1.f + expf(-z));
@@ -64,7 +90,7 @@ moe_route_kernel(const float* __restrict__ logits, int64_t stride, int experts, 
                 const float v = s_s[g * per + i];
                 if (v > a) { b = a; a = v; } else if (v > b) b = v;
             }
-            g_s[g] = per > 1 ? a + b : a;
+            g_s[g] = per > 1 && !choice ? a + b : a;
         }
         __syncthreads();
         for (int k = 0; k < group_keep; ++k) {
@@ -89,11 +115,18 @@ moe_route_kernel(const float* __restrict__ logits, int64_t stride, int experts, 
         if (lane == 0) {
             open_s[best] = 0;
             ids[t * top + k] = best;
-            weights[t * top + k] = softmax_top ? v : scale * v;
+            weights[t * top + k] = choice ? w_s[best] : softmax_top ? v : scale * v;
         }
         __syncthreads();
     }
-    if (softmax_top && lane == 0) {
+    if (choice) {
+        if (lane == 0) {
+            float sum = 0.f;
+            for (int k = 0; k < top; ++k) sum += weights[t * top + k];
+            sum += 1e-20f;
+            for (int k = 0; k < top; ++k) weights[t * top + k] /= sum;
+        }
+    } else if (softmax_top && lane == 0) {
         // the chosen logits, largest first: their softmax among themselves, summed in the order of the choice
         const float m = weights[t * top];
         float sum = 0.f;
@@ -112,7 +145,8 @@ moe_plan_kernel(const int32_t* __restrict__ ids, int64_t pairs, int experts, int
     __shared__ int count_s[MOE_MAX_EXPERTS], cursor_s[MOE_MAX_EXPERTS], begin_s[MOE_MAX_EXPERTS], tile0_s[MOE_MAX_EXPERTS];
     for (int e = threadIdx.x; e < experts; e += blockDim.x) count_s[e] = cursor_s[e] = 0;
     __syncthreads();
-    for (int64_t i = threadIdx.x; i < pairs; i += blockDim.x) atomicAdd(&count_s[ids[i]], 1);
+    for (int64_t i = threadIdx.x; i < pairs; i += blockDim.x)
+        if (ids[i] < experts) atomicAdd(&count_s[ids[i]], 1);      // (an identity takes no row of the products)
     __syncthreads();
     if (threadIdx.x == 0) {
         int at = 0, tiles = 0;
@@ -135,6 +169,7 @@ moe_plan_kernel(const int32_t* __restrict__ ids, int64_t pairs, int experts, int
     }
     for (int64_t i = threadIdx.x; i < pairs; i += blockDim.x) {
         const int e = ids[i];
+        if (e >= experts) { place[i] = -1; continue; }
         const int r = begin_s[e] + atomicAdd(&cursor_s[e], 1);
         place[i] = r;
         rows[r] = (int32_t)i;
@@ -332,13 +367,20 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(const T* __restrict__ o, int64_t o_stride, const int32_t* __restrict__ place,
                    const float* __restrict__ weights, int top, const T* __restrict__ add, int64_t add_stride,
+                   const float* __restrict__ add_gate, int64_t gate_stride, const T* __restrict__ x, int64_t x_stride,
                    T* __restrict__ y, int64_t y_stride, int width) {
     const int64_t t = blockIdx.y;
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= width) return;
     float sum = 0.f;
-    for (int c = 0; c < top; ++c) sum += weights[t * top + c] * to_float(o[(int64_t)place[t * top + c] * o_stride + i]);
-    if (add) sum += to_float(add[t * add_stride + i]);
+    for (int c = 0; c < top; ++c) {
+        const int at = place[t * top + c];
+        sum += weights[t * top + c] * to_float(at < 0 ? x[t * x_stride + i] : o[(int64_t)at * o_stride + i]);
+    }
+    if (add) {
+        const float a = to_float(add[t * add_stride + i]);
+        sum += add_gate ? a / (1.f + expf(-add_gate[t * gate_stride])) : a;
+    }
     y[t * y_stride + i] = from_float<T>(sum);
 }
 
@@ -349,11 +391,11 @@ NVA_EXPORT int NVA_NAME(nva_moe_route)(const float* logits, int64_t stride, int6
     if (tokens < 0 || tokens > 0x7fffffff || experts <= 0 || experts > MOE_MAX_EXPERTS)
         return nva_fail("moe_route: bad counts tokens=%lld experts=%d (up to %d)", (long long)tokens, experts, MOE_MAX_EXPERTS);
     if (group_count <= 0 || experts % group_count || group_keep <= 0 || group_keep > group_count || top <= 0 ||
-        top > group_keep * (experts / group_count))
+        top > group_keep * (experts / group_count) || softmax_top < 0 || softmax_top > 2)
         return nva_fail("moe_route: %d of %d experts in %d groups of which %d stay", top, experts, group_count, group_keep);
     if (!logits || !ids || !weights || stride < experts) return nva_fail("moe_route: a tensor is missing");
     hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)tokens), dim3(NVA_WAVE), 0, stream, logits, stride, experts, top,
-                       group_count, group_keep, scale, softmax_top ? 1 : 0, bias, ids, weights);
+                       group_count, group_keep, scale, softmax_top, bias, ids, weights);
     return nva_check_launch("moe_route");
 }
 
@@ -367,13 +409,15 @@ static int moe_tile_rows(int64_t pairs, int experts, int k, int ff) {
 }
 NVA_EXPORT int NVA_NAME(nva_moe_tile_rows)(int64_t pairs, int experts, int k, int ff) { return moe_tile_rows(pairs, experts, k, ff); }
 
+// ids from `experts` on are identities (x itself).  add_gate: float, one logit a token gate_stride apart, or null.
 // x [tokens, k] elements; ids, weights [tokens, top]; up [E * ff, k] (gated: [E * 2 ff, k], an expert's gate rows, then
 // its up rows), down [E * k, ff] elements; add [tokens, k] or null.
 // Scratch: place, rows int32 [tokens * top]; tiles int32 [3 * max_tiles + 1] with max_tiles = tokens * top / MOE_BM + E
 // (expert, first row, rows of every tile, then their number); hidden [tokens * top, ff], outs [tokens * top, k] elements.
 NVA_EXPORT int NVA_NAME(nva_moe_experts)(const void* x, int64_t x_stride, const int32_t* ids, const float* weights,
                                          int64_t tokens, int top, int experts, int k, int ff, const void* up,
-                                         const void* down, int act, int gated, const void* add, int64_t add_stride, int32_t* place,
+                                         const void* down, int act, int gated, const void* add, int64_t add_stride,
+                                         const float* add_gate, int64_t gate_stride, int32_t* place,
                                          int32_t* rows, int32_t* tiles, int64_t max_tiles, void* hidden, void* outs, void* y,
                                          int64_t y_stride, hipStream_t stream) {
     if (tokens == 0) return 0;
@@ -434,8 +478,9 @@ NVA_EXPORT int NVA_NAME(nva_moe_experts)(const void* x, int64_t x_stride, const 
         const unsigned nt = (unsigned)((tokens - t0) < 65535 ? (tokens - t0) : 65535);
         hipLaunchKernelGGL((moe_combine_kernel<elem_t>), dim3((k + 255) / 256, nt), dim3(256), 0, stream, (const elem_t*)outs,
                            (int64_t)k, place + t0 * top, weights + t0 * top, top,
-                           add ? (const elem_t*)add + t0 * add_stride : nullptr, add_stride, (elem_t*)y + t0 * y_stride,
-                           y_stride, k);
+                           add ? (const elem_t*)add + t0 * add_stride : nullptr, add_stride,
+                           add_gate ? add_gate + t0 * gate_stride : nullptr, gate_stride, (const elem_t*)x + t0 * x_stride,
+                           x_stride, (elem_t*)y + t0 * y_stride, y_stride, k);
     }
     return nva_check_launch("moe_experts");
 }

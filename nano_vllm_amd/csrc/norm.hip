@@ -248,6 +248,81 @@ NVA_EXPORT int NVA_NAME(nva_stream_rms_norm)(const void* a, int64_t a_stride, co
     return nva_check_launch("stream_rms_norm");
 }
 
+// ---------------------------------------------------------------------------- scaled addends, two norms of one stream
+// A block whose two sublayers read norms of their own of the same stream, and whose outputs are multiplied,
+// channel by channel, with learned vectors before they are added (layer scale):
+//     r <- r + sa * a + sb * b          (first: r <- a, unscaled: the embedding; a, b, sa, sb may each be absent)
+//     y1 = r * rsqrt(mean(r^2) + eps) * w1;   y2 = r * rsqrt(mean(r^2) + eps) * w2      (y2, w2 may be absent)
+// All arithmetic in float, each output rounded once.  One row sum serves both norms.  An addend may come as the
+// float partial sums of a split product.
+template <typename T>
+__global__ void __launch_bounds__(1024)
+stream_scaled_norm_kernel(const T* __restrict__ a, int64_t a_stride, PartialInput pa, const void* __restrict__ sa,
+                          const T* __restrict__ b, int64_t b_stride, PartialInput pb, const void* __restrict__ sb,
+                          int s_is_f32, float* residual, int64_t r_stride, int first,
+                          const void* __restrict__ w1, const void* __restrict__ w2, int w_is_f32,
+                          T* __restrict__ y1, T* __restrict__ y2, int64_t y_stride, int width, float eps) {
+    __shared__ float scratch[16];
+    const int64_t row = blockIdx.x;
+    const T* ar = a ? a + row * a_stride : nullptr;
+    const T* br = b ? b + row * b_stride : nullptr;
+    float* rr = residual + row * r_stride;
+    auto vec = [&](const void* v, int is_f32, int i) -> float {
+        return !v ? 1.f : is_f32 ? static_cast<const float*>(v)[i] : to_float(static_cast<const T*>(v)[i]);
+    };
+    constexpr int KEEP = 4;
+    float kept[KEEP];
+    float ss = 0.f;
+    int n = 0;
+    const bool adds = ar || br || pa.sums || pb.sums;
+    for (int i = threadIdx.x; i < width; i += blockDim.x, ++n) {
+        float s = first ? 0.f : rr[i];
+        float add = 0.f;
+        if (pa.sums) add = partial_value<T>(pa, row, width, i) * vec(sa, s_is_f32, i);
+        else if (ar) add = to_float(ar[i]) * vec(sa, s_is_f32, i);
+        if (pb.sums) add += partial_value<T>(pb, row, width, i) * vec(sb, s_is_f32, i);
+        else if (br) add += to_float(br[i]) * vec(sb, s_is_f32, i);
+        s += add;
+        if (adds || first) rr[i] = s;
+        if (n < KEEP) kept[n] = s;
+        ss += s * s;
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = rsqrtf(ss / (float)width + eps);
+    n = 0;
+    for (int i = threadIdx.x; i < width; i += blockDim.x, ++n) {
+        const float s = (n < KEEP ? kept[n] : rr[i]) * scale;
+        y1[row * y_stride + i] = from_float<T>(s * vec(w1, w_is_f32, i));
+        if (y2) y2[row * y_stride + i] = from_float<T>(s * vec(w2, w_is_f32, i));
+    }
+}
+
+// a, b: elements [rows, width], partial sums, or null; sa, sb: vectors [width] (float when s_is_f32, else elements) or
+// null (1); residual float [rows, width] in place; y1 and (optional) y2 [rows, width] with rows y_stride apart.
+NVA_EXPORT int NVA_NAME(nva_stream_scaled_norm)(const void* a, int64_t a_stride, const float* a_sums, int a_splits,
+                                                int64_t a_split_stride, const void* a_bias, const void* sa, const void* b,
+                                                int64_t b_stride, const float* b_sums, int b_splits, int64_t b_split_stride,
+                                                const void* b_bias, const void* sb, int s_is_f32, float* residual,
+                                                int64_t r_stride, int first, const void* w1, const void* w2, int w_is_f32,
+                                                void* y1, void* y2, int64_t y_stride, int64_t rows, int width, float eps,
+                                                hipStream_t stream) {
+    if (rows == 0) return 0;
+    if (rows < 0 || rows > 0x7fffffff || width <= 0)
+        return nva_fail("stream_scaled_norm: bad shape rows=%lld width=%d", (long long)rows, width);
+    if (!residual || !y1 || !w1 || (y2 && !w2)) return nva_fail("stream_scaled_norm: residual, output and weight are needed");
+    if (first && !a && !a_sums) return nva_fail("stream_scaled_norm: the stream starts with an addend");
+    const PartialInput pa{a_sums, a_splits, a_split_stride, a_bias}, pb{b_sums, b_splits, b_split_stride, b_bias};
+    if ((a_sums && (a_splits <= 0 || a_split_stride < rows * (int64_t)width)) ||
+        (b_sums && (b_splits <= 0 || b_split_stride < rows * (int64_t)width)))
+        return nva_fail("stream_scaled_norm: bad partial sums");
+    const int threads = (a_sums || b_sums) && rows <= 64 && width >= 1024 ? 1024
+                        : width >= 2048 ? 512 : width >= 1024 ? 256 : width >= 256 ? 128 : 64;
+    hipLaunchKernelGGL((stream_scaled_norm_kernel<elem_t>), dim3((unsigned)rows), dim3(threads), 0, stream,
+                       (const elem_t*)a, a_stride, pa, sa, (const elem_t*)b, b_stride, pb, sb, s_is_f32, residual, r_stride,
+                       first, w1, w2, w_is_f32, (elem_t*)y1, (elem_t*)y2, y_stride, width, eps);
+    return nva_check_launch("stream_scaled_norm");
+}
+
 // ---------------------------------------------------------------------------- a normed addend into the float stream
 // A sublayer's output enters the stream through a norm of its own and a constant, and the stream is normed
 // for the next sublayer, all in one pass over the row:

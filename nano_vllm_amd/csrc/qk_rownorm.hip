@@ -17,6 +17,12 @@
 // Cache layout: K [pages, Hkv, page, D], V [pages, Hkv, page / vt, DV, vt] (common.h).
 // With per_head the two norms run over every head by itself, mean over its D entries, with weights of D
 // entries that the heads share.
+// rot_interleaved: the rotation pairs the neighbours (2i, 2i + 1) of the first R channels instead of (i, i + R/2);
+// the table's row is the same (R/2 cosines, then R/2 sines, of the angles p * f_i).
+// v_norm: every value head is divided by its root mean square over DV (eps inside the root, no weight).
+// v_first_out, float [tokens, Hkv * DV]: the values as they are after the norm are also written there, unrounded (the
+// first of the layers that mix values hands them to the later ones of the same step).  v_first_in with v_mix (one
+// float read on the device): v <- (1 - v_mix) v + v_mix v_first_in, after the norm, before the store.
 // One workgroup per token.
 #include "common.h"
 
@@ -28,7 +34,9 @@ qk_rownorm_store_kernel(const T* __restrict__ qkv, int64_t stride, PartialInput 
                         const int32_t* __restrict__ positions, float temp_coef, int temp_every,
                         const float* __restrict__ rot_table, int rot,
                         const int32_t* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                        int page_size, int per_head) {
+                        int page_size, int per_head, int rot_interleaved, int v_norm,
+                        const float* __restrict__ v_first_in, const float* __restrict__ v_mix,
+                        float* __restrict__ v_first_out) {
     extern __shared__ __attribute__((aligned(16))) float row_s[];      // the token's row, as float; then a scale per head
     __shared__ float scratch[16];
     const int64_t t = blockIdx.x;
@@ -46,6 +54,17 @@ qk_rownorm_store_kernel(const T* __restrict__ qkv, int64_t stride, PartialInput 
         if (i < qd) sq += x * x; else if (i < qd + kd) sk += x * x;
     }
     float* const head_scale = row_s + width;                           // [num_heads + num_kv_heads], with per_head
+    float* const v_scale = head_scale + (per_head ? num_heads + num_kv_heads : 0);      // [num_kv_heads], with v_norm
+    if (v_norm) {
+        __syncthreads();
+        const int wave = tid / NVA_WAVE, lane = tid % NVA_WAVE, nwaves = blockDim.x / NVA_WAVE;
+        for (int g = wave; g < num_kv_heads; g += nwaves) {
+            float ss = 0.f;
+            for (int d = lane; d < v_dim; d += NVA_WAVE) ss += row_s[qd + kd + g * v_dim + d] * row_s[qd + kd + g * v_dim + d];
+            ss = wave_sum(ss);
+            if (lane == 0) v_scale[g] = rsqrtf(ss / (float)v_dim + eps);
+        }
+    }
     if (per_head) {
         __syncthreads();
         const int wave = tid / NVA_WAVE, lane = tid % NVA_WAVE, nwaves = blockDim.x / NVA_WAVE;
@@ -75,6 +94,12 @@ qk_rownorm_store_kernel(const T* __restrict__ qkv, int64_t stride, PartialInput 
         if (per_head && w) scale *= head_scale[(at + i) / head_dim];   // (at is a multiple of the head size)
         const float x = row_s[at + i] * scale * weight_of(w, per_head ? d : i);
         if (!rot_row || d >= rot) return x;
+        if (rot_interleaved) {
+            const int j = (d & 1) ? i - 1 : i + 1;
+            const float y = row_s[at + j] * scale * weight_of(w, per_head ? j % head_dim : j);
+            const float c = rot_row[d >> 1], sn = rot_row[half + (d >> 1)];
+            return (d & 1) ? x * c + y * sn : x * c - y * sn;
+        }
         const int f = d < half ? d : d - half;
         const int j = d < half ? i + half : i - half;
         const float y = row_s[at + j] * scale * weight_of(w, per_head ? j % head_dim : j);
@@ -82,6 +107,16 @@ qk_rownorm_store_kernel(const T* __restrict__ qkv, int64_t stride, PartialInput 
         return d < half ? x * c - y * sn : x * c + y * sn;
     };
     for (int i = tid; i < qd; i += blockDim.x) qrow[i] = from_float<T>(prepared(0, i, q_scale, q_weight));
+    if (v_norm) __syncthreads();                                      // (the values' scales; without per_head no barrier came since)
+    const float lam = v_first_in ? v_mix[0] : 0.f;
+    auto value_of = [&](int i) -> float {
+        float v = row_s[qd + kd + i];
+        if (v_norm) v *= v_scale[i / v_dim];
+        if (v_first_in) v = (1.f - lam) * v + lam * v_first_in[t * vd + i];
+        return v;
+    };
+    if (v_first_out)                                                  // also for a token that stores nothing
+        for (int i = tid; i < vd; i += blockDim.x) v_first_out[t * vd + i] = row_s[qd + kd + i] * (v_norm ? v_scale[i / v_dim] : 1.f);
     if (!kd || slot < 0 || !k_cache) return;
     const float k_scale = k_weight && !per_head ? rsqrtf(sk / (float)kd + eps) : 1.f;
     const int page = slot / page_size, off = slot % page_size;
@@ -94,7 +129,7 @@ qk_rownorm_store_kernel(const T* __restrict__ qkv, int64_t stride, PartialInput 
     for (int i = tid; i < vd; i += blockDim.x) {
         const int g = i / v_dim, d = i % v_dim;
         v_cache[((int64_t)page * num_kv_heads + g) * v_dim * (int64_t)page_size + nva_v_offset(off, d, v_dim, vt)] =
-            from_float<T>(row_s[qd + kd + i]);
+            from_float<T>(value_of(i));
     }
 }
 
@@ -111,7 +146,8 @@ NVA_EXPORT int NVA_NAME(nva_qk_rownorm_store)(const void* qkv, int64_t stride, c
                                               int w_is_f32, float eps, const int32_t* positions, float temp_coef,
                                               int temp_every, const float* rot_table, int rot, const int32_t* slots,
                                               void* k_cache, void* v_cache, int page_size, int per_head,
-                                              hipStream_t stream) {
+                                              int rot_interleaved, int v_norm, const float* v_first_in,
+                                              const float* v_mix, float* v_first_out, hipStream_t stream) {
     if (tokens == 0) return 0;
     if (tokens < 0 || tokens > 0x7fffffff) return nva_fail("qk_rownorm_store: bad token count %lld", (long long)tokens);
     if (num_heads <= 0 || num_kv_heads < 0 || head_dim <= 0 || v_dim <= 0)
@@ -129,10 +165,11 @@ NVA_EXPORT int NVA_NAME(nva_qk_rownorm_store)(const void* qkv, int64_t stride, c
         return nva_fail("qk_rownorm_store: a query temperature needs positions and a positive step");
     if (rot_table && (rot <= 0 || rot % 2 || rot > head_dim))
         return nva_fail("qk_rownorm_store: %d rotated channels of a head of %d", rot, head_dim);
+    if (v_first_in && (!v_mix || v_first_out)) return nva_fail("qk_rownorm_store: mixing values needs the factor, and reads or writes the first values, not both");
     if ((k_cache || v_cache) && (!k_cache || !v_cache || !slots || page_size <= 0 || !num_kv_heads))
         return nva_fail("qk_rownorm_store: storing needs both caches, the slots and the page size");
     auto kernel = qk_rownorm_store_kernel<elem_t>;
-    const size_t lds = (size_t)(width + (per_head ? num_heads + num_kv_heads : 0)) * sizeof(float);
+    const size_t lds = (size_t)(width + (per_head ? num_heads + num_kv_heads : 0) + (v_norm ? num_kv_heads : 0)) * sizeof(float);
     static bool raised = false;
     if (!raised && lds > 48 * 1024) {
         if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
@@ -145,7 +182,7 @@ NVA_EXPORT int NVA_NAME(nva_qk_rownorm_store)(const void* qkv, int64_t stride, c
     hipLaunchKernelGGL(kernel, dim3((unsigned)tokens), dim3(threads), lds, stream, (const elem_t*)qkv, stride, part,
                        (elem_t*)q_out, q_stride, num_heads, num_kv_heads, head_dim, v_dim, q_weight, k_weight, w_is_f32, eps,
                        positions, temp_coef, temp_every, rot_table, rot_table ? rot : 0, slots, (elem_t*)k_cache, (elem_t*)v_cache, page_size,
-                       per_head ? 1 : 0);
+                       per_head ? 1 : 0, rot_interleaved ? 1 : 0, v_norm ? 1 : 0, v_first_in, v_mix, v_first_out);
     return nva_check_launch("qk_rownorm_store");
 }
 

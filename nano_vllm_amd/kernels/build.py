@@ -41,6 +41,7 @@ MODULES: Dict[str, Tuple[str, Tuple[Optional[str], ...]]] = {
     "ssd": ("ssd.hip", ("bf16", "f32")),
     "moe": ("moe.hip", ("bf16", "f32")),
     "delta": ("delta.hip", ("bf16", "f32")),
+    "latent": ("latent.hip", ("bf16", "f32")),
 }
 
 _HEADERS = ("common.h",)

@@ -25,7 +25,7 @@ _LAST_ERROR_SYMBOL = {
     "attn_prefill": "nva_attn_prefill_last_error", "gemm_tile": "nva_gemm_tile_last_error",
     "qk_rownorm": "nva_qk_rownorm_last_error", "retention": "nva_retention_last_error",
     "ssd": "nva_ssd_last_error", "moe": "nva_moe_last_error",
-    "delta": "nva_delta_last_error",
+    "delta": "nva_delta_last_error", "latent": "nva_latent_last_error",
 }
 
 _loaded: Dict[Tuple[str, Optional[str]], ctypes.CDLL] = {}

@@ -477,6 +477,65 @@ class HipKernels:
                      self._stream())
         return out, residual
 
+    def stream_scaled_norm(self, addends, residual: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                           weight2: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                           out2: Optional[torch.Tensor] = None, dtype: Optional[torch.dtype] = None):
+        """Two norms of one float32 stream, and addends that enter it through a vector each:
+        residual <- residual + sum of scale_i * addend_i, in place (residual None: a new stream that starts as the
+        one addend, which then has no scale); y = residual * rsqrt(mean(residual^2) + eps) * weight, and y2 the
+        same with weight2 where that is given; all in float, each rounded once.  addends: up to two pairs
+        (tensor of the element type or a split product, vector [width] or None).  dtype: the outputs' element
+        type where neither an addend nor an output tensor says it.  Returns (y, y2 or None, residual)."""
+        pairs = [(a if isinstance(a, SplitSum) and self.fuse_split_sums else _t(a), s) for a, s in addends]
+        if len(pairs) > 2 or (residual is None and len(pairs) != 1):
+            raise KernelError("stream_scaled_norm: one or two addends (none with a stream that exists, one to start it)")
+        ref = pairs[0][0] if pairs else None
+        rows, width = (ref.shape if ref is not None else residual.shape)
+        elem = ref.dtype if ref is not None else out.dtype if out is not None else dtype
+        if elem is None:
+            raise KernelError("stream_scaled_norm: without addends the output tensor or dtype says the element type")
+        device = ref.device if ref is not None else residual.device
+        scale_f32 = None
+        args = []
+        for a, sc in pairs:
+            if tuple(a.shape) != (rows, width) or a.dtype != elem:
+                raise KernelError("stream_scaled_norm: the addends differ in shape or type")
+            if sc is not None:
+                f = self._norm_weight(sc, width, a)
+                if scale_f32 not in (None, f):
+                    raise KernelError("stream_scaled_norm: the two scale vectors differ in type")
+                scale_f32 = f
+            if isinstance(a, SplitSum):
+                args += [None, c_i64(0), _p(a.sums), c_i32(a.splits), c_i64(rows * width), _p(a.bias), _p(sc)]
+            else:
+                _, _, as_ = _rows2d(a, "stream_scaled_norm addend")
+                args += [_p(a), c_i64(as_), None, c_i32(0), c_i64(0), None, _p(sc)]
+        for _ in range(2 - len(pairs)):
+            args += [None, c_i64(0), None, c_i32(0), c_i64(0), None, None]
+        first = residual is None
+        if first:
+            if pairs[0][1] is not None:
+                raise KernelError("stream_scaled_norm: the addend that starts a stream has no scale")
+            residual = torch.empty((rows, width), dtype=torch.float32, device=device)
+        rrows, rw, rs = _rows2d(residual, "stream_scaled_norm residual")
+        if (rrows, rw) != (rows, width) or residual.dtype != torch.float32:
+            raise KernelError("stream_scaled_norm: the residual stream must be float32 of the addends' shape")
+        if out is None:
+            out = torch.empty((rows, width), dtype=elem, device=device)
+        if weight2 is not None and out2 is None:
+            out2 = torch.empty((rows, width), dtype=elem, device=device)
+        for o in (out, out2):
+            if o is not None and (tuple(o.shape) != (rows, width) or o.dtype != elem or not o.is_contiguous()):
+                raise KernelError("stream_scaled_norm: an output does not match")
+        wf = self._norm_weight(weight, width, out)
+        if weight2 is not None and self._norm_weight(weight2, width, out) != wf:
+            raise KernelError("stream_scaled_norm: the two weights differ in type")
+        library.call("norm", _suffix(out), "nva_stream_scaled_norm", *args, c_i32(scale_f32 or 0), _p(residual), c_i64(rs),
+                     c_i32(1 if first else 0), _p(weight), _p(weight2), c_i32(wf), _p(out),
+                     _p(out2) if weight2 is not None else None, c_i64(width), c_i64(rows), c_i32(width), c_f32(eps),
+                     self._stream())
+        return out, (out2 if weight2 is not None else None), residual
+
     def _stream_post_norm(self, addend, residual: torch.Tensor, weight: torch.Tensor, eps: float,
                           out: Optional[torch.Tensor] = None):
         """residual <- residual + mult * a / sqrt(mean(a^2) + eps_a) * w_a, then the stream's own norm, in one pass;
@@ -598,32 +657,40 @@ class HipKernels:
         return out
 
     # ------------------------------------------------------------------ routed feed-forward
+    ROUTINGS = {"sigmoid_groups": 0, "softmax_top": 1, "softmax_choice": 2}
+
     def moe_route(self, logits: torch.Tensor, top: int, group_count: int, group_keep: int, scale: float,
                   routing: str = "sigmoid_groups", bias: Optional[torch.Tensor] = None):
         """From the router's float32 logits [tokens, experts]: int32 [tokens, top] experts and float32
         [tokens, top] weights (scale * sigmoid score).  Experts form group_count groups of neighbours; a
         group's score is the sum of its two largest scores; only experts of the group_keep best groups are
         chosen, the `top` with the largest scores.  routing "softmax_top": the `top` largest logits (plus the
-        float32 bias [experts], if any) are chosen and weighted by the softmax over the chosen alone."""
+        float32 bias [experts], if any) are chosen and weighted by the softmax over the chosen alone.  routing
+        "softmax_choice": scores s = softmax(logits) over all experts; chosen by s + bias, within the group_keep groups
+        whose largest s + bias is largest; weights s of the chosen over their sum (+ 1e-20).  logits may be the leading
+        columns of wider rows."""
         rows, experts, ls = _rows2d(logits, "router logits")
         if logits.dtype != torch.float32:
             raise KernelError("moe_route: the logits must be float32")
-        if routing not in ("sigmoid_groups", "softmax_top"):
+        if routing not in self.ROUTINGS:
             raise KernelError(f"moe_route: unknown routing {routing!r}")
         if bias is not None and (bias.dtype != torch.float32 or tuple(bias.shape) != (experts,) or not bias.is_contiguous()):
             raise KernelError(f"moe_route: the bias must be contiguous float32 [{experts}]")
         ids = torch.empty((rows, top), dtype=torch.int32, device=logits.device)
         weights = torch.empty((rows, top), dtype=torch.float32, device=logits.device)
         library.call("moe", self.suffix, "nva_moe_route", _p(logits), c_i64(ls), c_i64(rows), c_i32(experts), c_i32(top),
-                     c_i32(group_count), c_i32(group_keep), c_f32(scale), c_i32(1 if routing == "softmax_top" else 0),
+                     c_i32(group_count), c_i32(group_keep), c_f32(scale), c_i32(self.ROUTINGS[routing]),
                      _p(bias), _p(ids), _p(weights), self._stream())
         return ids, weights
 
     def moe_experts(self, x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, up: torch.Tensor, down: torch.Tensor,
-                    num_experts: int, act: str = "relu2", add=None, gated: bool = False) -> torch.Tensor:
+                    num_experts: int, act: str = "relu2", add=None, gated: bool = False,
+                    add_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
         """y[t] = sum over the choices c of weights[t, c] * act(x[t] Wu_e^T) Wd_e^T with e = ids[t, c] (+ add[t]).
         up [E * ff, k] and down [E * k, ff] hold the experts' matrices one below the other.  gated: up is
-        [E * 2 ff, k], an expert's gate rows and then its up rows, and the hidden layer act(x Wg_e^T) * (x Wu_e^T)."""
+        [E * 2 ff, k], an expert's gate rows and then its up rows, and the hidden layer act(x Wg_e^T) * (x Wu_e^T).
+        An id from num_experts on is an identity: its output is x[t] itself.  add_gate, float32 [tokens] (a column of
+        wider rows may be given): add[t] is multiplied by sigmoid(add_gate[t])."""
         if act not in self.PLAIN_ACTIVATIONS:
             raise KernelError(f"moe_experts: unknown activation {act!r}")
         x = _t(x)
@@ -645,6 +712,11 @@ class HipKernels:
             arows, aw, add_stride = _rows2d(add, "moe addend")
             if (arows, aw) != (tokens, k) or add.dtype != x.dtype:
                 raise KernelError("moe_experts: the addend does not match the input")
+        gate_stride = 0
+        if add_gate is not None:
+            if add is None or add_gate.dtype != torch.float32 or add_gate.dim() != 1 or add_gate.shape[0] != tokens:
+                raise KernelError("moe_experts: the addend's gate is float32 [tokens] and comes with an addend")
+            gate_stride = add_gate.stride(0)
         pairs = tokens * top
         tile_rows = getattr(library.load("moe", self.suffix), f"nva_moe_tile_rows_{self.suffix}")
         bm = int(tile_rows(c_i64(pairs), c_i32(num_experts), c_i32(k), c_i32(ff)))
@@ -655,7 +727,7 @@ class HipKernels:
         y = torch.empty((tokens, k), dtype=x.dtype, device=x.device)
         library.call("moe", _suffix(x), "nva_moe_experts", _p(x), c_i64(xs), _p(ids), _p(weights), c_i64(tokens), c_i32(top),
                      c_i32(num_experts), c_i32(k), c_i32(ff), _p(up), _p(down), c_i32(self.PLAIN_ACTIVATIONS[act]),
-                     c_i32(1 if gated else 0), _p(add), c_i64(add_stride), _p(ints[:pairs]), _p(ints[pairs:2 * pairs]), _p(ints[2 * pairs:]), c_i64(max_tiles),
+                     c_i32(1 if gated else 0), _p(add), c_i64(add_stride), _p(add_gate), c_i64(gate_stride), _p(ints[:pairs]), _p(ints[pairs:2 * pairs]), _p(ints[2 * pairs:]), c_i64(max_tiles),
                      _p(hidden), _p(outs), _p(y), c_i64(k), self._stream())
         return y
 
@@ -1150,8 +1222,14 @@ class HipKernels:
                          positions: Optional[torch.Tensor], temp_coef: float, temp_every: int,
                          slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                          v_cache: Optional[torch.Tensor], rot_table: Optional[torch.Tensor] = None,
-                         norm_per_head: bool = False) -> torch.Tensor:
-        """norm_per_head: the two norms run over every head by itself, with weights [head_dim] that the heads share.
+                         norm_per_head: bool = False, rot_interleaved: bool = False, v_norm: bool = False,
+                         v_first_in: Optional[torch.Tensor] = None, v_mix: Optional[torch.Tensor] = None,
+                         v_first_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """rot_interleaved: the rotation pairs the neighbours (2i, 2i + 1).  v_norm: every value head divided by its root
+        mean square (eps, no weight).  v_first_out, float32 [tokens, kv_heads * v_head_dim]: receives the values after the
+        norm.  v_first_in (the same shape) with v_mix (float32, one number on the device): v <- (1 - v_mix) v + v_mix
+        v_first_in before the store.
+        norm_per_head: the two norms run over every head by itself, with weights [head_dim] that the heads share.
         rot_table, float32 [tokens, rot]: after norm and temperature the first rot channels of every head
         of q and k are rotated in pairs (i, i + rot / 2) by the token's row (rot / 2 cosines, then sines).
         q and k normed over the whole projection (all heads at once, plain weights [heads * head_dim]
@@ -1190,6 +1268,13 @@ class HipKernels:
         if k_cache is not None:
             page_size = self._check_cache(k_cache, v_cache, num_kv_heads, head_dim, qkv.dtype, v_head_dim)
             _i32(slots, tokens, "slots")
+        vd = num_kv_heads * v_head_dim
+        for name, vf in (("v_first_in", v_first_in), ("v_first_out", v_first_out)):
+            if vf is not None and (vf.dtype != torch.float32 or tuple(vf.shape) != (tokens, vd) or not vf.is_contiguous()):
+                raise KernelError(f"qk_rownorm_store: {name} must be contiguous float32 [{tokens}, {vd}]")
+        if v_first_in is not None and (v_mix is None or v_mix.dtype != torch.float32 or v_mix.numel() != 1 or
+                                       v_first_out is not None):
+            raise KernelError("qk_rownorm_store: mixing values needs one float32 factor, and reads or writes the first values")
         if partial:
             # the projection's partial sums (and bias) are added up by the kernel; q gets a tensor of its own
             q = torch.empty((tokens, num_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
@@ -1202,7 +1287,9 @@ class HipKernels:
                      c_i32(num_heads), c_i32(num_kv_heads), c_i32(head_dim), c_i32(v_head_dim), _p(q_weight), _p(k_weight),
                      c_i32(wf), c_f32(eps), _p(positions), c_f32(float(temp_coef)), c_i32(int(temp_every) if temp_coef else 1),
                      _p(rot_table), c_i32(rot), _p(slots), _p(k_cache), _p(v_cache), c_i32(page_size),
-                     c_i32(1 if norm_per_head and q_weight is not None else 0), self._stream())
+                     c_i32(1 if norm_per_head and q_weight is not None else 0), c_i32(1 if rot_interleaved else 0),
+                     c_i32(1 if v_norm else 0), _p(v_first_in), _p(v_mix) if v_first_in is not None else None,
+                     _p(v_first_out), self._stream())
         return q
 
     def sigmoid_mul(self, x: torch.Tensor, gate: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -1239,8 +1326,11 @@ class HipKernels:
                         k_cache: torch.Tensor, v_cache: torch.Tensor, batch, group: int, scale: float,
                         window: Optional[int] = None, out: Optional[torch.Tensor] = None,
                         v_head_dim: Optional[int] = None, sinks: Optional[torch.Tensor] = None,
-                        chunk: Optional[int] = None, softcap: Optional[float] = None, keep_first: int = 0) -> torch.Tensor:
-        """chunk: a query at position p reads the keys from floor(p / chunk) * chunk on only.
+                        chunk: Optional[int] = None, softcap: Optional[float] = None, keep_first: int = 0,
+                        sigmoid_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """sigmoid_bias, float32 [heads]: no softmax; a visible key weighs sigmoid(score + sigmoid_bias[head]), and the
+        weights are not normalised over the keys.
+        chunk: a query at position p reads the keys from floor(p / chunk) * chunk on only.
         softcap: a score s (after the scale) becomes softcap * tanh(s / softcap).  keep_first (with a window):
         every query also reads the first keep_first positions of its sequence, however far back.
         Causal attention of the step's tokens over the cache.  `batch` is the step's
@@ -1281,7 +1371,11 @@ class HipKernels:
         keep = int(keep_first) if window and keep_first else 0
         if cap < 0.0 or keep < 0:
             raise KernelError("attention: a negative softcap or number of kept positions")
-        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and v_dim == head_dim
+        if sigmoid_bias is not None and (sigmoid_bias.dtype != torch.float32 or sigmoid_bias.shape != (num_heads,) or
+                                         not sigmoid_bias.is_contiguous() or sinks is not None):
+            raise KernelError(f"attention: sigmoid_bias must be contiguous float32 [{num_heads}] and goes without sinks")
+        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and v_dim == head_dim \
+            and sigmoid_bias is None
         if batch.num_decode > 0 and mfma and \
                 self._decode_kernel_takes(num_heads // num_kv_heads, head_dim, page_size, q, qs, out, os_):
             start = batch.num_decode
@@ -1297,7 +1391,7 @@ class HipKernels:
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
                          c_i32(chunk or 0), c_i32(keep), c_f32(cap), _p(sinks), _p(self.fault_flag), self._stream())
             tokens = batch.num_decode            # what is left: the single tokens before the portions, if any
-        if self.tiled_general_attention and start <= batch.num_decode < tokens and not window and \
+        if self.tiled_general_attention and start <= batch.num_decode < tokens and not window and sigmoid_bias is None and \
                 max(head_dim, v_dim) <= GENERAL_TILED_MAX_HEAD_DIM:
             # portions of prompts in float arithmetic: the per-token kernel's arithmetic, operation for
             # operation, with the keys staged once for 32 query rows
@@ -1316,16 +1410,63 @@ class HipKernels:
             reach = min(x for x in (batch.max_kv_len, (window + keep) if window else None, chunk) if x)
             # (Only where a cap or kept positions keep bfloat16 tokens from the matrix-core decode kernel: everywhere
             # else this kernel's sums keep the one order that the tiled form for portions shares, bit for bit.)
-            shared = self.shared_general_attention and q.dtype == torch.bfloat16 and (cap > 0.0 or keep > 0)
+            shared = self.shared_general_attention and q.dtype == torch.bfloat16 and (cap > 0.0 or keep > 0) and \
+                sigmoid_bias is None
             shares = max(1, min(16, reach // 128, 4096 // (n * num_heads))) if shared else 1
             part = torch.empty(n * num_heads * shares * (2 + v_dim), dtype=torch.float32, device=q.device) if shares > 1 else None
             library.call("attn_generic", _suffix(q), "nva_paged_attention_generic", _p(q[start:start + n]), c_i64(qs),
                          _p(out[start:]), c_i64(os_), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
                          _p(batch.token_seq[start:]), _p(batch.positions[start:]), c_i64(n), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(v_dim), c_i32(page_size), c_f32(scale),
-                         c_i32(window or 0), c_i32(chunk or 0), c_i32(keep), c_f32(cap), _p(sinks), _p(part), c_i32(shares),
+                         c_i32(window or 0), c_i32(chunk or 0), c_i32(keep), c_f32(cap), _p(sinks), _p(sigmoid_bias), _p(part), c_i32(shares),
                          _p(self.fault_flag), self._stream())
         return out
+
+    # ------------------------------------------------------------------ attention through a latent
+    def latent_prepare(self, proj: torch.Tensor, heads: int, dim: int, rot: int, rank: int, weight: torch.Tensor, eps: float,
+                       rot_table: torch.Tensor, slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                       v_cache: Optional[torch.Tensor]) -> torch.Tensor:
+        """proj [tokens, heads * (dim + rot) + rank + rot]: per head [dim plain | rot turned] query entries, then the
+        token's raw latent and its raw turned key part.  The latent is normed (weight, eps), the turned parts are
+        rotated in pairs of neighbours by rot_table (float32 [tokens, rot]: cosines, then sines); the cache's key row
+        of the token becomes [latent | turned key part], its value row the latent.  Returns q2 [tokens, heads *
+        (rank + rot)] with every head's turned part in its last rot entries; the first rank are left for the caller."""
+        proj = _t(proj)
+        tokens, width, stride = _rows2d(proj, "latent projection")
+        if width != heads * (dim + rot) + rank + rot:
+            raise KernelError(f"latent_prepare: a row of {width} is not heads * (dim + rot) + rank + rot")
+        if rot_table.dtype != torch.float32 or tuple(rot_table.shape) != (tokens, rot) or not rot_table.is_contiguous():
+            raise KernelError(f"latent_prepare: the rotation table must be contiguous float32 [{tokens}, {rot}]")
+        wf = self._norm_weight(weight, rank, proj)
+        page_size = 0
+        if k_cache is not None:
+            page_size = self._check_cache(k_cache, v_cache, 1, rank + rot, proj.dtype, rank)
+            _i32(slots, tokens, "slots")
+        q2 = torch.empty((tokens, heads * (rank + rot)), dtype=proj.dtype, device=proj.device)
+        library.call("latent", _suffix(proj), "nva_latent_prepare", _p(proj), c_i64(stride), c_i64(tokens), c_i32(heads),
+                     c_i32(dim), c_i32(rot), c_i32(rank), _p(weight), c_i32(wf), c_f32(eps), _p(rot_table), _p(q2),
+                     c_i64(q2.shape[1]), _p(slots), _p(k_cache), _p(v_cache), c_i32(page_size), self._stream())
+        return q2
+
+    def heads_linear(self, x: torch.Tensor, x_head: int, w: torch.Tensor, heads: int, n_out: int, k_in: int,
+                     transposed: bool, y: torch.Tensor, y_head: int, y_offset: int = 0) -> torch.Tensor:
+        """A product per head: y[t, h * y_head + y_offset + n] = sum_k W[h][n][k] x[t, h * x_head + k], n < n_out, k < k_in.
+        w is contiguous [heads * n_out, k_in], or with transposed [heads * k_in, n_out] (W[h][n][k] = w[h * k_in + k, n]).
+        x and y are 2-d with rows of any stride.  Float sums over k in ascending order, rounded once."""
+        x = _t(x)
+        tokens, xw, xs = _rows2d(x, "heads_linear input")
+        yrows, yw, ys = _rows2d(y, "heads_linear output")
+        if yrows != tokens or y.dtype != x.dtype or w.dtype != x.dtype or not w.is_contiguous() or \
+                tuple(w.shape) != ((heads * k_in, n_out) if transposed else (heads * n_out, k_in)):
+            raise KernelError("heads_linear: the output or the matrices do not fit the input")
+        if (heads - 1) * x_head + k_in > xw or (heads - 1) * y_head + y_offset + n_out > yw or x_head < 0 or y_head < 0:
+            raise KernelError("heads_linear: the heads do not fit the rows")
+        w_n, w_k = (1, n_out) if transposed else (k_in, 1)
+        yv = y[:, y_offset:] if y_offset else y
+        library.call("latent", _suffix(x), "nva_heads_linear", _p(x), c_i64(xs), c_i64(x_head), _p(w), c_i64(n_out * k_in),
+                     c_i64(w_n), c_i64(w_k), _p(yv), c_i64(ys), c_i64(y_head), c_i64(tokens), c_i32(heads), c_i32(n_out),
+                     c_i32(k_in), self._stream())
+        return y
 
     # ------------------------------------------------------------------ delta rule
     def channel_delta(self, proj: torch.Tensor, decay_in: torch.Tensor, gate_in: torch.Tensor, heads: int, kv_heads: int,

@@ -26,6 +26,14 @@ Options beyond the reference's attention, each a parameter:
     gate "sigmoid"                  the heads' outputs are multiplied, entry by entry, with sigmoid(x Wg^T)
                                     before the output projection; Wg [heads * v_head_dim, hidden] is packed
                                     below q, k and v into the one projection
+    v_norm                          every value head is divided by its root mean square (eps inside the root, no
+                                    weight) before it is cached
+    v_mix (a name)                  the layers of a model that give the same name mix their values: the first of them
+                                    in the order keeps its values of the step's tokens (after the norm), every later
+                                    one caches (1 - lam) v + lam v_first, lam a learned number of its own
+    weights "sigmoid"               no softmax: a visible key weighs sigmoid(score + b_head), b a learned number per
+                                    head, and the weights are not normalised over the keys
+An encoding that says `interleaved` rotates the neighbours (2i, 2i + 1) instead of the pairs (i, i + R/2).
 With values of their own size (or whole-projection norms, or a temperature) the position encoding's
 rotation is applied by the same preparation kernel, from the cosines and sines of the step's tokens
 (position_encoding.step_table): such a model needs no table of all positions.
@@ -54,8 +62,9 @@ class Attention(Part):
     qk_norm_scope ("head" | "projection"), q_temperature (None or {"coef", "every"}), sink (bool),
     chunk (None or positions), o_bias (bool), step_rotation (bool: rotate from the step's own table
     also where the per-head kernel could serve), softcap (None or a positive number), keep_first (positions),
-    sink_value (None or a number), gate (None or "sigmoid"), and the names of the checkpoint tensors (q_name, ...,
-    q_norm_name, k_norm_name, sink_name, g_name)."""
+    sink_value (None or a number), gate (None or "sigmoid"), v_norm (bool), v_mix (None or a name shared by the layers
+    that mix), weights ("softmax" | "sigmoid"), and the names of the checkpoint tensors (q_name, ..., q_norm_name,
+    k_norm_name, sink_name, g_name, v_mix_name, score_bias_name)."""
 
     def __init__(self, params: Mapping, build: BuildContext):
         super().__init__(params, build)
@@ -108,12 +117,26 @@ class Attention(Part):
         if self.gate not in (None, "sigmoid"):
             raise ValueError(f"attention: gate must be 'sigmoid' or absent, got {self.gate!r}")
         self.g_name = p.get("g_name", "g_proj")
+        self.v_norm = bool(p.get("v_norm", False))
+        self.v_mix = p.get("v_mix")
+        self.v_mix_name = p.get("v_mix_name", "v_mix")
+        self.weighting = p.get("weights", "softmax")
+        if self.weighting not in ("softmax", "sigmoid"):
+            raise ValueError(f"attention: weights must be 'softmax' or 'sigmoid', got {self.weighting!r}")
+        self.score_bias_name = p.get("score_bias_name", "score_bias")
+        if self.weighting == "sigmoid" and (self.sink or self.sink_value is not None or self.softcap is not None
+                                            or self.keep_first or self.chunk is not None):
+            raise ValueError("attention: sigmoid weights go without sink, softcap, kept positions and chunks")
+        if (self.v_norm or self.v_mix) and self.shared:
+            raise ValueError("attention: a value norm or mixed values go with a cache of the run's own")
+        self.interleaved = bool(getattr(build.position_encodings.get(p.get("position_encoding")), "interleaved", False))
         self._device = build.device
         self._sink_tensor = None
         # The whole-projection preparation has its own kernel, which also scales q by its temperature
         # and stores values of their own size; the per-head one rotates.  Each does what its model needs.
         self.row_prepare = self.norm_scope == "projection" or self.temp_coef != 0.0 or self.v_head_dim != self.head_dim \
-            or bool(p.get("step_rotation", False)) or self.gate is not None
+            or bool(p.get("step_rotation", False)) or self.gate is not None or self.v_norm or bool(self.v_mix) \
+            or self.interleaved
         if self.row_prepare and self.position_encoding is not None and not hasattr(self.position_encoding, "step_table"):
             raise ValueError("attention: with whole-projection norms, a query temperature or values of their own "
                              "size the position encoding must offer step_table")
@@ -124,7 +147,7 @@ class Attention(Part):
     def kernel_modules(self):
         prepare = "qk_rownorm" if self.row_prepare else "rope"
         rope = ("rope",) if self.row_prepare and self.position_encoding else ()
-        if self.v_head_dim != self.head_dim:
+        if self.v_head_dim != self.head_dim or self.weighting == "sigmoid":
             return (prepare, "attn_generic") + rope
         return (prepare, "attn_generic", "attn_decode", "attn_prefill") + \
             (("rope",) if self.row_prepare and self.position_encoding else ())
@@ -156,6 +179,10 @@ class Attention(Part):
                                                sources=(Source(f"{self.k_norm_name}.weight", 0, kn),))
         if self.sink:
             d["sinks"] = ParamDecl((self.heads,), dtype="float32", sources=(Source(self.sink_name, 0, self.heads),))
+        if self.v_mix:
+            d[self.v_mix_name] = ParamDecl((), dtype="float32")        # (one number: the tensor goes by its own name)
+        if self.weighting == "sigmoid":
+            d["score_bias"] = ParamDecl((self.heads,), dtype="float32", sources=(Source(self.score_bias_name, 0, self.heads),))
         d[f"{self.o_name}.weight"] = ParamDecl((h, self.heads * self.v_head_dim))
         if self.o_bias:
             d[f"{self.o_name}.bias"] = ParamDecl((h,))
@@ -201,6 +228,20 @@ class Attention(Part):
             extra = {"rot_table": pe.step_table(batch)} if pe is not None else {}
             if self.qk_norm and self.norm_scope == "head":
                 extra["norm_per_head"] = True
+            if self.interleaved:
+                extra["rot_interleaved"] = True
+            if self.v_norm:
+                extra["v_norm"] = True
+            if self.v_mix:
+                # the first layer of the name to run in a step leaves its values for the others
+                kept = batch.step_cache
+                first = kept.get(("v_first", self.v_mix))
+                if first is None:
+                    first = kept[("v_first", self.v_mix)] = torch.empty(
+                        (x.shape[0], self.kv_heads * self.v_head_dim), dtype=torch.float32, device=x.device)
+                    extra["v_first_out"] = first
+                else:
+                    extra["v_first_in"], extra["v_mix"] = first, w[self.v_mix_name]
             q = k.qk_rownorm_store(qkv, self.heads, kv_heads, self.head_dim, self.v_head_dim, qw, kw, self.eps,
                                    batch.positions, self.temp_coef, self.temp_every, slots, kc, vc, **extra)
         elif pe is None or table is not None:
@@ -222,6 +263,8 @@ class Attention(Part):
         if self.keep_first:
             extra["keep_first"] = self.keep_first
         sinks = self._sinks()
+        if self.weighting == "sigmoid":
+            extra["sigmoid_bias"] = w["score_bias"]
         if sinks is not None or self.v_head_dim != self.head_dim:
             o = k.paged_attention(q, self.heads, self.kv_heads, self.head_dim, cache.k, cache.v, batch, cache.group,
                                   self.scale, self.window, v_head_dim=self.v_head_dim, sinks=sinks, **extra)

@@ -56,6 +56,14 @@ class NormedAddend:
 
 
 @dataclass
+class ScaledAddend:
+    """A sublayer's output on its way into a float32 residual stream through a learned vector: the stream
+    takes x * scale, channel by channel (layer scale).  The norm that follows adds it while it reads the stream."""
+    x: object                         # [rows, width] of the element type (or a product left as partial sums)
+    scale: torch.Tensor               # [width]
+
+
+@dataclass
 class BuildContext:
     """What a part may use while it is built."""
     kernels: object                   # the operations (kernels.ops.HipKernels or a stand-in of the same methods)

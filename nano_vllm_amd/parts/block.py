@@ -17,6 +17,11 @@ The residual stream r is float32 whatever the element type.  The sum is deferred
 norm as well: the block returns the two sublayer outputs as a list of addends with the stream as
 it was before them, and the next block's norm (or the model's final norm) adds them.  The first
 block gets the embedding as its one addend.  A layer may have no feed-forward.
+With a part in the role "feed_forward_norm" the feed-forward reads a norm of its own of the same stream
+(x = norm(r), y = feed_forward_norm(r), both made in one pass over r), and with layer_scale = True the
+two outputs are multiplied, channel by channel, by learned vectors of the block's own before they are added:
+    r <- r + (s1 * mixer(x) + s2 * feed_forward(y))
+(the vectors' names in the checkpoint: mixer_scale_name, feed_forward_scale_name).
 
 "sandwich_residual": a norm before and a norm after every sublayer, the normed output times a
 constant added to the stream:
@@ -36,7 +41,7 @@ from typing import Dict, Mapping
 
 import torch
 
-from .base import BuildContext, NormedAddend, Part
+from .base import BuildContext, NormedAddend, ParamDecl, Part, ScaledAddend
 from .registry import make_part, register_part
 
 
@@ -93,7 +98,9 @@ class PreNormResidualBlock(Part):
 
 
 class ParallelResidualBlock(Part):
-    ROLES = ("norm", "mixer", "feed_forward")
+    """params: layer_scale (bool), mixer_scale_name, feed_forward_scale_name; parts and names by role: norm, mixer,
+    and optionally feed_forward and feed_forward_norm."""
+    ROLES = ("norm", "mixer", "feed_forward_norm", "feed_forward")
 
     def __init__(self, params: Mapping, build: BuildContext):
         super().__init__(params, build)
@@ -105,10 +112,31 @@ class ParallelResidualBlock(Part):
         self.norm = make_part("norm", parts["norm"], build)
         self.mixer = make_part("mixer", parts["mixer"], build)
         self.feed_forward = make_part("feed_forward", parts["feed_forward"], build) if parts.get("feed_forward") else None
+        self.feed_forward_norm = None
+        if parts.get("feed_forward_norm"):
+            if self.feed_forward is None:
+                raise ValueError("parallel_residual block: a feed-forward norm without a feed-forward")
+            self.feed_forward_norm = make_part("norm", parts["feed_forward_norm"], build)
+            if getattr(self.feed_forward_norm, "offset", 0.0) or getattr(self.norm, "offset", 0.0) or \
+                    self.feed_forward_norm.eps != self.norm.eps:
+                raise ValueError("parallel_residual block: two norms of one stream share their eps and have plain weights")
+        self.layer_scale = bool(params.get("layer_scale", False))
+        self.mixer_scale_name = params.get("mixer_scale_name", "mixer_scale")
+        self.feed_forward_scale_name = params.get("feed_forward_scale_name", "feed_forward_scale")
+        self.width = build.hidden_size
+        self.dtype = build.dtype
         self._children = {names[r]: getattr(self, r) for r in self.ROLES if getattr(self, r) is not None}
 
     def children(self) -> Dict[str, Part]:
         return self._children
+
+    def param_decls(self):
+        if not self.layer_scale:
+            return {}
+        d = {self.mixer_scale_name: ParamDecl((self.width,), dtype="stored32", init="norm")}
+        if self.feed_forward is not None:
+            d[self.feed_forward_scale_name] = ParamDecl((self.width,), dtype="stored32", init="norm")
+        return d
 
     def cache_need(self):
         return self.mixer.cache_need()
@@ -117,13 +145,23 @@ class ParallelResidualBlock(Part):
     def replays_state_steps(self):
         return self.mixer.replays_state_steps
 
+    def _out(self, x, scale_name):
+        return ScaledAddend(x, self.weights[scale_name]) if self.layer_scale else x
+
     def forward(self, h, residual, batch, cache):
         addends = h if isinstance(h, (tuple, list)) else (h,)
-        x, residual = self.norm.forward_add(addends, residual)
-        a = self.mixer.forward(x, batch, cache)
+        if self.feed_forward_norm is not None:
+            x, y, residual = self.kernels.stream_scaled_norm(
+                [(a.x, a.scale) if hasattr(a, "scale") else (a, None) for a in addends], residual,
+                self.norm.weights["weight"], self.norm.eps, weight2=self.feed_forward_norm.weights["weight"],
+                dtype=self.dtype)
+        else:
+            x, residual = self.norm.forward_add(addends, residual)
+            y = x
+        a = self._out(self.mixer.forward(x, batch, cache), self.mixer_scale_name)
         if self.feed_forward is None:
             return (a,), residual
-        return (a, self.feed_forward.forward(x, batch)), residual
+        return (a, self._out(self.feed_forward.forward(y, batch), self.feed_forward_scale_name)), residual
 
 
 class SandwichResidualBlock(Part):

@@ -8,6 +8,7 @@ with an offset, and every norm that is handed a list of addends instead of one t
 residual stream kept in float32: the stream takes the sum of the addends, the norm is computed in
 float and rounded once to the element type.  An addend may be a NormedAddend (parts.base): a sublayer's
 output that enters the stream through a norm of its own and a constant factor; the same pass does both norms.
+Or a ScaledAddend: an output that is multiplied, channel by channel, by a learned vector on its way into the stream.
 
 "dynamic_tanh": y = tanh(alpha * x) * weight + bias with one learned number alpha per norm: no mean,
 no variance, every entry by itself.  It works on a float32 residual stream (a list of addends, as
@@ -44,6 +45,13 @@ class RMSNorm(Part):
         """residual <- x + residual; returns (norm(residual), residual).  x may be a list of one or
         two addends: the residual is then a float32 stream (None: it starts as their sum)."""
         if isinstance(x, (tuple, list)):
+            if any(hasattr(a, "scale") for a in x):
+                if self.offset != 0.0:
+                    raise ValueError("rms_norm: scaled addends go with a plain weight")
+                y, _, residual = self.kernels.stream_scaled_norm(
+                    [(a.x, a.scale) if hasattr(a, "scale") else (a, None) for a in x], residual, self.weights["weight"],
+                    self.eps, out=out)
+                return y, residual
             return self.kernels.stream_rms_norm(tuple(x), residual, self.weights["weight"], self.eps, self.offset, out=out)
         if self.offset != 0.0:
             raise ValueError("rms_norm: a weight offset goes with a float32 residual stream (a list of addends)")

@@ -35,5 +35,5 @@ def known_parts(role: str):
 
 
 def _load_builtin() -> None:
-    from . import (norm, rotary, attention, retention, state_space, channel_delta, side_by_side, feed_forward, experts, block,  # noqa: F401
+    from . import (norm, rotary, attention, latent_attention, retention, state_space, channel_delta, side_by_side, feed_forward, experts, block,  # noqa: F401
                    embedding)

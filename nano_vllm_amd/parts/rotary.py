@@ -18,6 +18,7 @@ A mixer whose model names no longest sequence asks for step_table(batch) instead
 positions: the cosines and sines of the step's own tokens, [tokens, R], made once per step by a
 kernel that reads the positions on the device (so a captured step makes it anew at every replay) and
 shared by all the layers that rotate alike.
+"rotary_interleaved": the same angles, the pairs being the neighbours (2i, 2i + 1) of the first R channels.
 "none": no encoding.
 """
 from __future__ import annotations
@@ -78,6 +79,16 @@ class RotaryNeox(Part):
         raise NotImplementedError("rotary_neox is applied through its table")
 
 
+class RotaryInterleaved(RotaryNeox):
+    """The same angles p * theta^(-2i/R), i < R/2, over the first R channels of a head, but the pair that turns by
+    angle i is the neighbours (2i, 2i + 1).  Offered through step_table only (the cosines and sines of the step's
+    tokens, R/2 cosines and then R/2 sines a row): the mixers' preparation kernels pair the channels."""
+    interleaved = True
+
+    def rotary_table(self):
+        return None
+
+
 class NoPositionEncoding(Part):
     def rotary_table(self):
         return None
@@ -87,4 +98,5 @@ class NoPositionEncoding(Part):
 
 
 register_part("position_encoding", "rotary_neox", RotaryNeox)
+register_part("position_encoding", "rotary_interleaved", RotaryInterleaved)
 register_part("position_encoding", "none", NoPositionEncoding)

@@ -97,6 +97,29 @@ class TorchKernels:
             return out, residual
         return y, residual
 
+    def stream_scaled_norm(self, addends, residual, weight, eps, weight2=None, out=None, out2=None, dtype=None):
+        """The float32 stream takes every addend times its vector; one or two norms of it, each rounded once."""
+        dt = out.dtype if out is not None else dtype
+        add = None
+        for a, sc in addends:
+            dt = a.dtype
+            x = a.float() * (sc.float() if sc is not None else 1.0)
+            add = x if add is None else add + x
+        if residual is None:
+            residual = add.clone()
+        elif add is not None:
+            residual += add
+        unit = residual * torch.rsqrt(residual.pow(2).mean(-1, keepdim=True) + eps)
+        y = (unit * weight.float()).to(dt)
+        y2 = (unit * weight2.float()).to(dt) if weight2 is not None else None
+        if out is not None:
+            out.copy_(y)
+            y = out
+        if out2 is not None and y2 is not None:
+            out2.copy_(y2)
+            y2 = out2
+        return y, y2, residual
+
     def stream_dyt(self, addends, residual, weight, bias, alpha, out=None):
         """The float32 stream takes the sum of the addends; tanh(alpha * stream) * weight + bias, rounded once."""
         add = None
@@ -155,6 +178,18 @@ class TorchKernels:
             z = logits.float() + (bias.float() if bias is not None else 0.0)
             best = z.topk(top, dim=-1)
             return best.indices.to(torch.int32), torch.softmax(best.values, dim=-1)
+        if routing == "softmax_choice":
+            s = torch.softmax(logits.float(), dim=-1)
+            choice = s + (bias.float() if bias is not None else 0.0)
+            per = E // group_count
+            grouped = choice.view(T, group_count, per)
+            kept = grouped.max(-1).values.topk(group_keep, dim=-1).indices
+            allowed = torch.zeros((T, group_count), dtype=torch.bool, device=logits.device)
+            allowed.scatter_(1, kept, True)
+            masked = grouped.masked_fill(~allowed[:, :, None], float("-inf")).view(T, E)
+            ids = masked.topk(top, dim=-1).indices
+            w = s.gather(1, ids)
+            return ids.to(torch.int32), (w / (w.sum(-1, keepdim=True) + 1e-20)).float()
         s = torch.sigmoid(logits.float())
         per = E // group_count
         grouped = s.view(T, group_count, per)
@@ -166,7 +201,7 @@ class TorchKernels:
         ids = masked.topk(top, dim=-1).indices
         return ids.to(torch.int32), (s.gather(1, ids) * scale).float()
 
-    def moe_experts(self, x, ids, weights, up, down, num_experts, act="relu2", add=None, gated=False):
+    def moe_experts(self, x, ids, weights, up, down, num_experts, act="relu2", add=None, gated=False, add_gate=None):
         """sum over a token's experts e of weight * act(x Wu_e^T) Wd_e^T (+ add); up [E * ff, K], down [E * K, ff].
         gated: up [E * 2 ff, K] holds an expert's gate rows, then its up rows, and the hidden layer is
         act(x Wg_e^T) * (x Wu_e^T)."""
@@ -185,8 +220,11 @@ class TorchKernels:
                 h = self._activation((x[rows].float() @ up[e * ff:(e + 1) * ff].float().T), act).to(x.dtype).float()
                 y = (h @ down[e * K:(e + 1) * K].float().T).to(x.dtype).float()
                 out[rows] += (weights * hit)[rows].sum(-1, keepdim=True) * y
+        identity = ids >= num_experts               # such a choice gives the token's input back
+        if bool(identity.any()):
+            out += (weights * identity).sum(-1, keepdim=True) * x.float()
         if add is not None:
-            out += add.float()
+            out += add.float() * (torch.sigmoid(add_gate.float())[:, None] if add_gate is not None else 1.0)
         return out.to(x.dtype)
 
     # feed-forward (activation.py:8-11)
@@ -275,7 +313,8 @@ class TorchKernels:
         return torch.cat((ang.cos(), ang.sin()), dim=-1)
 
     def qk_rownorm_store(self, qkv, num_heads, num_kv_heads, head_dim, v_head_dim, q_weight, k_weight, eps,
-                         positions, temp_coef, temp_every, slots, k_cache, v_cache, rot_table=None, norm_per_head=False):
+                         positions, temp_coef, temp_every, slots, k_cache, v_cache, rot_table=None, norm_per_head=False,
+                         rot_interleaved=False, v_norm=False, v_first_in=None, v_mix=None, v_first_out=None):
         """q and k normed over the whole projection, q times its position's temperature, both rotated by
         the rows of rot_table (one per token: cosines, then sines, for the first channels of a head),
         k and v stored."""
@@ -289,6 +328,10 @@ class TorchKernels:
             R = rot_table.shape[1]
             x = x.reshape(T, heads, head_dim)
             cos, sin = rot_table[:, None, : R // 2], rot_table[:, None, R // 2:]
+            if rot_interleaved:
+                a, b = x[..., 0:R:2], x[..., 1:R:2]
+                pairs = torch.stack((a * cos - b * sin, b * cos + a * sin), dim=-1).reshape(T, heads, R)
+                return torch.cat((pairs, x[..., R:]), dim=-1).reshape(T, heads * head_dim)
             a, b = x[..., : R // 2], x[..., R // 2:R]
             return torch.cat((a * cos - b * sin, b * cos + a * sin, x[..., R:]), dim=-1).reshape(T, heads * head_dim)
         def normed(x, heads, w):
@@ -308,6 +351,15 @@ class TorchKernels:
             if k_weight is not None:
                 k = normed(k, num_kv_heads, k_weight)
             qkv[:, qd:qd + kd] = turn(k, num_kv_heads).to(dt)
+            v = qkv[:, qd + kd:].float()
+            if v_norm:
+                v = v.reshape(T, num_kv_heads, v_head_dim)
+                v = (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, num_kv_heads * v_head_dim)
+            if v_first_out is not None:
+                v_first_out.copy_(v)
+            if v_first_in is not None:
+                v = (1.0 - v_mix.float()) * v + v_mix.float() * v_first_in
+            qkv[:, qd + kd:] = v.to(dt)
             if k_cache is not None:
                 page_size, vt = k_cache.shape[2], v_cache.shape[4]
                 s = slots.long()
@@ -449,7 +501,8 @@ class TorchKernels:
 
     # attention (attention.py:64-75): token by token through the block table
     def paged_attention(self, q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, batch, group, scale,
-                        window=None, out=None, v_head_dim=None, sinks=None, chunk=None, softcap=None, keep_first=0):
+                        window=None, out=None, v_head_dim=None, sinks=None, chunk=None, softcap=None, keep_first=0,
+                        sigmoid_bias=None):
         T = q.shape[0]
         D, G = head_dim, num_heads // num_kv_heads
         DV = v_head_dim or head_dim
@@ -476,7 +529,9 @@ class TorchKernels:
                 s = (keys[:, h // G] @ qt[h]) * scale
                 if softcap:
                     s = softcap * torch.tanh(s / softcap)
-                if sinks is not None:       # one more term in the denominator: a key without a value
+                if sigmoid_bias is not None:   # every key by itself, no normalisation
+                    p = torch.sigmoid(s + sigmoid_bias[h].float())
+                elif sinks is not None:       # one more term in the denominator: a key without a value
                     p = torch.softmax(torch.cat((s, sinks[h:h + 1].float())), dim=0)[:-1]
                 else:
                     p = torch.softmax(s, dim=0)
@@ -485,6 +540,39 @@ class TorchKernels:
         if out is not None:
             out.copy_(y)
             return out
+        return y
+
+    # attention through a latent
+    def latent_prepare(self, proj, heads, dim, rot, rank, weight, eps, rot_table, slots, k_cache, v_cache):
+        T = proj.shape[0]
+        dt = proj.dtype
+        qd = heads * (dim + rot)
+        cos, sin = rot_table[:, : rot // 2], rot_table[:, rot // 2:]
+
+        def turn(x):                                    # [..., rot] with the tokens first
+            a, b = x[..., 0::2], x[..., 1::2]
+            c, s = (cos, sin) if x.dim() == 2 else (cos[:, None], sin[:, None])
+            return torch.stack((a * c - b * s, b * c + a * s), dim=-1).reshape(x.shape)
+        q = proj[:, :qd].float().reshape(T, heads, dim + rot)
+        q2 = torch.zeros((T, heads, rank + rot), dtype=dt, device=proj.device)
+        q2[:, :, rank:] = turn(q[:, :, dim:]).to(dt)
+        if k_cache is not None:
+            c = proj[:, qd:qd + rank].float()
+            c = (c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * weight.float()).to(dt)
+            kr = turn(proj[:, qd + rank:].float()).to(dt)
+            page_size, vt = k_cache.shape[2], v_cache.shape[4]
+            s = slots.long()
+            ok = s >= 0
+            page, off = s[ok] // page_size, s[ok] % page_size
+            k_cache[page, 0, off, :] = torch.cat((c, kr), dim=-1)[ok]
+            v_cache[page, 0, off // vt, :, off % vt] = c[ok]
+        return q2.reshape(T, heads * (rank + rot))
+
+    def heads_linear(self, x, x_head, w, heads, n_out, k_in, transposed, y, y_head, y_offset=0):
+        wh = w.float().reshape(heads, k_in, n_out).transpose(1, 2) if transposed else w.float().reshape(heads, n_out, k_in)
+        for h in range(heads):
+            xh = x[:, h * x_head: h * x_head + k_in].float()
+            y[:, h * y_head + y_offset: h * y_head + y_offset + n_out] = (xh @ wh[h].T).to(y.dtype)
         return y
 
     # sampling (sampler.py:8-12), same counter-based noise as the kernel
