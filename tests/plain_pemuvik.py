@@ -59,6 +59,8 @@ def silu(z):
 
 def turn_pairs(x, rot, first_position=0):
     """x [T, heads, dim]: neighbouring channels (2i, 2i + 1) below rot["dims"] turned by the token's position."""
+    if not rot:
+        return x
     R = rot["dims"]
     out = x.clone()
     for t in range(x.shape[0]):
@@ -103,7 +105,7 @@ def window_attention(h, m, w, p, eps, shared):
     T = h.shape[0]
     q = (h @ w[p + "q"].T + w[p + "q.b"]).view(T, m["heads"], m["dim"])
     k = (h @ w[p + "k"].T + w[p + "k.b"]).view(T, m["kv_heads"], m["dim"])
-    q, k = turn_pairs(q, m["rot"]), turn_pairs(k, m["rot"])
+    q, k = turn_pairs(q, m.get("rot")), turn_pairs(k, m.get("rot"))
     v = window_values(h, m, w, p, eps, shared)
     o = sigmoid_window_attend(q, k, v, m, w[p + "pb"])
     return o @ w[p + "o"].T + w[p + "o.b"]
