@@ -36,6 +36,12 @@ beside Nozurax and Qwen3 at equal layer sizes.
 does the same for the Kirisun design (layers of the channel-wise delta rule and of a gated window attention in
 turn, each with a routed feed-forward of gated experts whose chosen experts add up to the dense layer's inner
 size), beside Mafarax and Qwen3 at equal layer sizes.
+
+    python bench.py --design pemuvik [--design-sizes 1024,2048,4096] [--layers 4]
+
+does the same for the Pemuvik design (layers of a window attention with sigmoid weights and a routed feed-forward,
+and of an attention through a shared latent and a dense feed-forward, in turn), beside Kirisun and Qwen3 at equal
+layer sizes.
 """
 import argparse
 import json
@@ -67,7 +73,7 @@ def parse_args():
                     help="context of one more decode point at the default batch (0: none)")
     ap.add_argument("--serve-seqs", type=int, default=256,
                     help="requests of the reference's benchmark workload through LLM.generate (0: not run)")
-    ap.add_argument("--design", default=None, choices=["nozurax", "mafarax", "kirisun"],
+    ap.add_argument("--design", default=None, choices=["nozurax", "mafarax", "kirisun", "pemuvik"],
                     help="measure this design beside Qwen3 at equal layer sizes instead of the default workload")
     ap.add_argument("--design-sizes", default="1024,2048,4096", help="model widths of the --design measurement")
     ap.add_argument("--design-alone", action="store_true", help="the --design measurement without the models beside it "
@@ -101,11 +107,26 @@ def kirisun_config(width: int, layers: int, dtype: str) -> dict:
     return _kirisun(layers, width, heads, kv, dim, dim, inner, DESIGN_VOCAB, window=1024, dtype=dtype)
 
 
+def pemuvik_config(width: int, layers: int, dtype: str) -> dict:
+    """A Pemuvik model of the width's layer sizes: window-attention layers with the dense model's heads (keys and values
+    of 128, a window of 1024 positions, half the head rotated, sigmoid weights) with 30 gated experts of an eighth of the
+    dense inner size and 2 identity outputs of which a token runs 8, beside a shared expert of a quarter of it, and
+    latent-attention layers in turn (as many heads, 128 plain and 64 rotated query entries a head, a latent of 384) with
+    the dense gated layer."""
+    from nano_vllm_amd.models.shapes import _pemuvik
+    heads, kv, dim, inner = DESIGN_SIZES[width]
+    return _pemuvik(layers, width, heads, kv, dim, dim, inner, DESIGN_VOCAB, window=1024, dtype=dtype, experts=30, group_count=4,
+                    group_keep=2)
+
+
 def design_configs(width: int, layers: int, dtype: str, design: str = "nozurax"):
     """config.json of a Nozurax model and of the Qwen3 model with the same layer sizes (and, for the Mafarax
     measurement, of the Mafarax model first)."""
     if design == "mafarax":
         return {"mafarax": mafarax_config(width, layers, dtype), **design_configs(width, layers, dtype)}
+    if design == "pemuvik":
+        return {"pemuvik": pemuvik_config(width, layers, dtype), "kirisun": kirisun_config(width, layers, dtype),
+                "qwen3": design_configs(width, layers, dtype)["qwen3"]}
     if design == "kirisun":
         return {"kirisun": kirisun_config(width, layers, dtype), "mafarax": mafarax_config(width, layers, dtype),
                 "qwen3": design_configs(width, layers, dtype)["qwen3"]}

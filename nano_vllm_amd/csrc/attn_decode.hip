@@ -206,7 +206,7 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
                    const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
                    const int32_t* __restrict__ block_tables, int table_stride, int tokens, int max_segments,
                    int num_q_heads, int num_kv_heads, int page_size, float scale, float softcap,
-                   const float* __restrict__ sinks, int32_t* error_flag) {
+                   const float* __restrict__ sinks, const float* __restrict__ sig_bias, int32_t* error_flag) {
     constexpr int KP = D / 32;          // 16-byte pieces of a key row per lane = MFMAs per S tile
     constexpr int DT = D / 16;          // 16-channel tiles of the output
     const int lane = threadIdx.x, col = lane & 15, g = lane >> 4;
@@ -287,8 +287,11 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
     f32x4 acc[DT];
 #pragma unroll
     for (int i = 0; i < DT; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY, l_run = 0.f;      // the maximum in units of raw scores
+    // sig_bias: no softmax; a visible key weighs sigmoid(scale s + sig_bias[head]) and nothing is normalised: the running
+    // maximum stays at zero (nothing is rescaled, segments join with weight one) and the sum is not used.
+    float m_run = sig_bias ? 0.f : -INFINITY, l_run = 0.f;      // the maximum in units of raw scores
     const float c_exp = scale * 1.4426950408889634f;      // scale * log2(e)
+    const float sig_b2 = sig_bias ? sig_bias[kvh * G + (col < G ? col : 0)] * 1.4426950408889634f : 0.f;
     // a cap on the scores, in the raw scores' units: s <- (cap / scale) tanh(s scale / cap), tanh(y) = 1 - 2 / (1 + e^(2 y))
     const bool capped = softcap > 0.f;
     const float cap_in = capped ? 2.f * 1.4426950408889634f * scale / softcap : 0.f, cap_out = capped ? softcap / scale : 0.f;
@@ -341,7 +344,8 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
             s[i] = (key >= first && key < kv_len) ? raw : -INFINITY;
             m_new = fmaxf(m_new, s[i]);
         }
-        m_new = nva_max_over_rows(m_new);
+        if (sig_bias) m_new = m_run;
+        else m_new = nva_max_over_rows(m_new);
         // a head that has seen no key yet keeps -inf as its maximum; exponents then use a finite
         // stand-in so that -inf - (-inf) never arises
         const float m_use = fmaxf(m_new, -1e30f);
@@ -350,7 +354,8 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
         bf16x8 pf;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const __bf16 pb16 = (__bf16)__builtin_amdgcn_exp2f(fmaf(s[i], c_exp, neg_mc));
+            const __bf16 pb16 = sig_bias ? (__bf16)__builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-fmaf(s[i], c_exp, sig_b2)))
+                                         : (__bf16)__builtin_amdgcn_exp2f(fmaf(s[i], c_exp, neg_mc));
             pf[i] = pb16;
             psum += (float)pb16;           // the sum of what the product below really uses
         }
@@ -373,7 +378,7 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
         if (rec.w == 1) {
             // a sink: one more term exp(sink) in the denominator, in the units of the running maximum
             if (sinks) l_run += __builtin_amdgcn_exp2f(sinks[head] * 1.4426950408889634f - fmaxf(m_run, -1e30f) * c_exp);
-            const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+            const float inv = sig_bias ? 1.f : l_run > 0.f ? 1.f / l_run : 0.f;
             __bf16* orow = out + t * out_stride + (int64_t)head * D;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
@@ -421,7 +426,7 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
 __global__ void __launch_bounds__(MERGE_WAVES * NVA_WAVE)
 attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                          const int32_t* __restrict__ plan, __bf16* __restrict__ out, int64_t out_stride,
-                         int num_q_heads, int head_dim, const float* __restrict__ sinks) {
+                         int num_q_heads, int head_dim, const float* __restrict__ sinks, int plain_sum) {
     __shared__ float acc_s[MERGE_WAVES][4 * NVA_WAVE];
     __shared__ float l_s[MERGE_WAVES];
     const int64_t t = blockIdx.x;
@@ -463,7 +468,7 @@ attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restri
 #pragma unroll
     for (int w = 0; w < MERGE_WAVES; ++w) l += l_s[w];
     if (sinks) l += __expf(sinks[head] - m);              // the sink joins the denominator once, after the segments
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+    const float inv = plain_sum ? 1.f : l > 0.f ? 1.f / l : 0.f;     // (plain_sum: weights that are not normalised)
     __bf16* orow = out + t * out_stride + (int64_t)head * head_dim;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -480,7 +485,7 @@ attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restri
 __global__ void __launch_bounds__(MERGE_WAVES * NVA_WAVE)
 attn_decode_merge_wave_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                               const int32_t* __restrict__ plan, __bf16* __restrict__ out, int64_t out_stride,
-                              int tokens, int num_q_heads, int head_dim, const float* __restrict__ sinks) {
+                              int tokens, int num_q_heads, int head_dim, const float* __restrict__ sinks, int plain_sum) {
     const int lane = threadIdx.x % NVA_WAVE;
     const int64_t pair = (int64_t)blockIdx.x * MERGE_WAVES + threadIdx.x / NVA_WAVE;
     if (pair >= (int64_t)tokens * num_q_heads) return;
@@ -515,7 +520,7 @@ attn_decode_merge_wave_kernel(const float* __restrict__ part_o, const float* __r
             for (int i = 0; i < 4; ++i) acc[i] += v[j][i] * wj[j];
     }
     if (sinks) l += __expf(sinks[head] - m);
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+    const float inv = plain_sum ? 1.f : l > 0.f ? 1.f / l : 0.f;
     __bf16* orow = out + t * out_stride + (int64_t)head * head_dim;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -624,8 +629,8 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
                                     const int32_t* plan, const void* k_cache, const void* v_cache,
                                     const int32_t* block_tables, int table_stride, int64_t tokens, int num_q_heads,
                                     int num_kv_heads, int head_dim, int page_size, float scale, float softcap,
-                                    int max_segments, int waves, const float* sinks, int32_t* error_flag,
-                                    hipStream_t stream) {
+                                    int max_segments, int waves, const float* sinks, const float* sig_bias,
+                                    int32_t* error_flag, hipStream_t stream) {
     if (tokens == 0) return 0;
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads)
         return nva_fail("attn_decode: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
@@ -640,6 +645,7 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
                  "page_size %% 8 == 0 (got head_dim %d, group %d, page %d)", head_dim, G, page_size);
         return 1;
     }
+    if (sig_bias && (sinks || softcap > 0.f)) return nva_fail("attn_decode: sigmoid weights go without a sink and a cap");
     if (tokens < 0 || tokens > DEC_MAX_TOKENS || num_q_heads > 65535)
         return nva_fail("attn_decode: %lld tokens (at most %d a launch) or %d heads exceed the grid", (long long)tokens,
                         DEC_MAX_TOKENS, num_q_heads);
@@ -653,7 +659,7 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
     hipLaunchKernelGGL(attn_decode_kernel<DD>, dim3((unsigned)waves), dim3(NVA_WAVE), 0, stream, (const __bf16*)q, \
                        q_stride, (__bf16*)out, out_stride, part_o, part_ml, plan, (const __bf16*)k_cache,         \
                        (const __bf16*)v_cache, block_tables, table_stride, (int)tokens, max_segments, num_q_heads,  \
-                       num_kv_heads, page_size, scale, softcap, sinks, error_flag)
+                       num_kv_heads, page_size, scale, softcap, sinks, sig_bias, error_flag)
     switch (head_dim) {
         case 32: LAUNCH(32); break;
         case 64: LAUNCH(64); break;
@@ -674,12 +680,12 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
     if (pairs >= 2 * resident) {            // pairs enough for a wave each
         hipLaunchKernelGGL(attn_decode_merge_wave_kernel, dim3((unsigned)((pairs + MERGE_WAVES - 1) / MERGE_WAVES)),
                            dim3(MERGE_WAVES * NVA_WAVE), 0, stream, part_o, part_ml, plan, (__bf16*)out, out_stride,
-                           (int)tokens, num_q_heads, head_dim, sinks);
+                           (int)tokens, num_q_heads, head_dim, sinks, sig_bias ? 1 : 0);
         return nva_check_launch("attn_decode_merge");
     }
     dim3 mgrid((unsigned)tokens, (unsigned)num_q_heads);
     hipLaunchKernelGGL(attn_decode_merge_kernel, mgrid, dim3(MERGE_WAVES * NVA_WAVE), 0, stream, part_o, part_ml, plan,
-                       (__bf16*)out, out_stride, num_q_heads, head_dim, sinks);
+                       (__bf16*)out, out_stride, num_q_heads, head_dim, sinks, sig_bias ? 1 : 0);
     return nva_check_launch("attn_decode_merge");
 }
 

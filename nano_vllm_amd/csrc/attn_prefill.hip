@@ -95,7 +95,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
                     const int32_t* __restrict__ cu_seqlens_q, const int32_t* __restrict__ kv_lens,
                     const int32_t* __restrict__ tiles, int num_tiles, int paired, int num_q_heads, int num_kv_heads,
                     int page_size, float scale, int window, int key_chunk, int keep_first, float softcap,
-                    const float* __restrict__ sinks, int32_t* error_flag) {
+                    const float* __restrict__ sinks, const float* __restrict__ sig_bias, int32_t* error_flag) {
     constexpr int DC = D / 16;            // 16-channel steps of the first product
     constexpr int MT = D / 32;            // 32-channel tiles of the output
     constexpr int KR = D / 8;             // 16-byte pieces of a K row (one key)
@@ -188,7 +188,10 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     for (int i = 0; i < MT; ++i)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
+    // sig_bias: no softmax; a visible key weighs sigmoid(scale s + sig_bias[head]), nothing is normalised: the running
+    // maximum stays at zero, so nothing is ever rescaled, and the sum is not used.
+    float m_run = sig_bias ? 0.f : -INFINITY, l_run = 0.f;
+    const float sig_b2 = sig_bias ? sig_bias[head] * 1.4426950408889634f : 0.f;
 
     // S tile row r = col holds key 16*(a/2) + 8*h' + 4*(a%2) + b with a = r/8, h' = (r/4)%2, b = r%4
     const int a_r = col >> 3, h_r = (col >> 2) & 1, b_r = col & 3;
@@ -351,6 +354,17 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
                     const int key = kb + 32 * kt + 16 * (e >> 3) + 8 * h + (e & 7);
                     if (key > pos || (key < first_row && key >= keep)) s[kt][e] = -INFINITY;
                 }
+        }
+        if (sig_bias) {
+            // 1 / (1 + 2^-(s c + b)); a masked score of -inf gives 1 / inf = 0
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    pf[kt][e >> 3][e & 7] = (__bf16)__builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-fmaf(s[kt][e], c_exp, sig_b2)));
+            alpha = 1.f;
+            rescale = false;
+            return;
         }
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
@@ -551,7 +565,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     // a sink: one more term exp(sink) in the denominator (a key without a value), in the units of the
     // running maximum; it joins once, after the tiles (and after the sets of waves have met)
     if (sinks) l_run += __builtin_amdgcn_exp2f(sinks[head] * 1.4426950408889634f - fmaxf(m_run, -1e30f) * c_exp);
-    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+    const float inv = sig_bias ? 1.f : l_run > 0.f ? 1.f / l_run : 0.f;
     __bf16* orow = out + (int64_t)(q_begin + row) * out_stride + (int64_t)head * D;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -577,8 +591,8 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
                                      int table_stride, const int32_t* cu_seqlens_q, const int32_t* kv_lens,
                                      const int32_t* tiles, int64_t num_tiles, int num_q_heads,
                                      int num_kv_heads, int head_dim, int page_size, float scale, int window, int chunk,
-                                     int keep_first, float softcap, const float* sinks, int32_t* error_flag,
-                                     hipStream_t stream) {
+                                     int keep_first, float softcap, const float* sinks, const float* sig_bias,
+                                     int32_t* error_flag, hipStream_t stream) {
     if (num_tiles == 0) return 0;
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads)
         return nva_fail("attn_prefill: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
@@ -594,6 +608,7 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
     }
     const int G = num_q_heads / num_kv_heads;
     const int64_t grid_y = (int64_t)num_kv_heads * ((G + PF_WAVES - 1) / PF_WAVES);
+    if (sig_bias && (sinks || softcap > 0.f)) return nva_fail("attn_prefill: sigmoid weights go without a sink and a cap");
     if (keep_first < 0 || !(softcap >= 0.f) || !(softcap <= 3.0e38f))
         return nva_fail("attn_prefill: bad kept positions %d or cap %g", keep_first, (double)softcap);
     if (!tiles || num_tiles < 0 || num_tiles * grid_y > 0x7fffffff || window < 0 || chunk < 0 || table_stride <= 0)
@@ -620,7 +635,7 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
                        (const __bf16*)q, q_stride, (__bf16*)out, out_stride, (const __bf16*)k_cache,                 \
                        (const __bf16*)v_cache, block_tables, table_stride, cu_seqlens_q, kv_lens, tiles,             \
                        (int)num_tiles, SS == 1 && PF_WAVES_PER_SIMD(DD) == 2 && total <= 2 * cus ? (int)total : 0,   \
-                       num_q_heads, num_kv_heads, page_size, scale, window, chunk, keep_first, softcap, sinks, error_flag)
+                       num_q_heads, num_kv_heads, page_size, scale, window, chunk, keep_first, softcap, sinks, sig_bias, error_flag)
 #define LAUNCH(DD)                                                                                                 \
     do {                                                                                                           \
         if (PF_WAVES_PER_SIMD(DD) == 2 && two_sets) LAUNCH_SETS(DD, PF_WAVES_PER_SIMD(DD));                         \

@@ -154,4 +154,230 @@ NVA_EXPORT int NVA_NAME(nva_heads_linear)(const void* x, int64_t x_stride, int64
     return nva_check_launch("heads_linear");
 }
 
+#if defined(NVA_BF16)
+// ---------------------------------------------------------------------------- the attention itself, on the matrix cores
+// One key/value head for all query heads: the query heads of a token are the 16 columns of the products, so a key row
+// that is fetched serves all of them.  A wave takes one token, 16 of its heads and a share of its keys, in tiles of 32:
+//     S^T = K Q^T      K rows straight from the cache as the A operand (a lane 16 bytes of a key row), Q^T in registers
+//     O^T += V^T P^T   V^T from the value cache, which holds the latent transposed in tiles of 32 keys (a lane 2 x 8
+//                      bytes of a channel's row), P^T as the lanes hold it after the first product: the second
+//                      product's index over the keys is 8 g + j <-> key 4 g + j (j < 4) and 16 + 4 g + j - 4 (j >= 4)
+//                      of the tile, for both operands, so that nothing is exchanged between lanes
+// with an online softmax in float (exp2 with log2 e folded in), the sink as the first share's starting maximum with a
+// sum of one.  All tokens are treated alike, a prompt's and single ones (every row of a tile has the same position, so
+// only a token's last tile is masked).  With more than one share the shares leave (maximum, sum, unnormalised output)
+// and latent_attn_merge_kernel joins them in the order of the shares.
+typedef __attribute__((ext_vector_type(8))) __bf16 lat_bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 lat_bf16x4;
+typedef __attribute__((ext_vector_type(4))) float lat_f32x4;
+#define LAT_TILE 32
+#define LAT_MAX_ROT 128
+
+template <int MAXC>
+__global__ void __launch_bounds__(NVA_WAVE)
+latent_attn_kernel(const __bf16* __restrict__ q2, int64_t q_stride, __bf16* __restrict__ out, int64_t out_stride,
+                   float* __restrict__ part, const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
+                   const int32_t* __restrict__ block_tables, int table_stride, const int32_t* __restrict__ token_seq,
+                   const int32_t* __restrict__ positions, int heads, int rank, int rot, int page_size, float scale,
+                   const float* __restrict__ sinks, int32_t* error_flag) {
+    constexpr int KS = (MAXC + LAT_MAX_ROT) / 32;      // steps of 32 channels of the first product, at most
+    constexpr int CB = MAXC / 16;                      // blocks of 16 latent channels of the output, at most
+    const int64_t t = blockIdx.x;
+    const int share = blockIdx.y, shares = gridDim.y;
+    const int lane = threadIdx.x, col = lane & 15, g = lane >> 4;
+    const int head = blockIdx.z * 16 + col;
+    const bool head_ok = head < heads;
+    const int width = rank + rot;                      // a key row
+    const int steps = (width + 31) / 32, blocks = rank / 16;
+    const int pos = positions[t];
+    const int32_t* table = block_tables + (int64_t)token_seq[t] * table_stride;
+    const int tiles = pos / LAT_TILE + 1;
+    const int per = (tiles + shares - 1) / shares;
+    const int tile_lo = share * per, tile_hi = min(tiles, tile_lo + per);
+
+    lat_bf16x8 qf[KS];
+    const __bf16* qrow = q2 + t * q_stride + (int64_t)(head_ok ? head : 0) * width;
+#pragma unroll
+    for (int c = 0; c < KS; ++c) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[c][e] = (__bf16)0.f;
+        if (c < steps && head_ok && 32 * c + 8 * g < width) qf[c] = *reinterpret_cast<const lat_bf16x8*>(qrow + 32 * c + 8 * g);
+    }
+    lat_f32x4 acc[CB];
+#pragma unroll
+    for (int b = 0; b < CB; ++b) acc[b] = lat_f32x4{0.f, 0.f, 0.f, 0.f};
+    const bool with_sink = sinks && share == 0 && head_ok;
+    float m_run = with_sink ? sinks[head] : -INFINITY, l_run = with_sink ? 1.f : 0.f;      // of the scaled scores
+    const float log2e = 1.4426950408889634f;
+    const int tiles_per_page = page_size / LAT_TILE;
+
+    for (int tile = tile_lo; tile < tile_hi; ++tile) {
+        const int kb = tile * LAT_TILE;
+        int page = table[kb / page_size];
+        const bool no_page = page < 0;
+        if (no_page) {
+            if (error_flag && lane == 0) atomicOr(error_flag, 2);        // a visible key has no page
+            page = 0;
+        }
+        const int in_page = kb % page_size;
+        // ---- scores: rows of K as they lie, keys kb + col and kb + 16 + col
+        const __bf16* k0 = k_cache + ((int64_t)page * page_size + in_page + col) * width + 8 * g;
+        const __bf16* k1 = k0 + (int64_t)16 * width;
+        lat_f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < KS; ++c) {
+            if (c < steps) {
+                lat_bf16x8 ka, kc;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ka[e] = kc[e] = (__bf16)0.f;
+                if (32 * c + 8 * g < width) {
+                    ka = *reinterpret_cast<const lat_bf16x8*>(k0 + 32 * c);
+                    kc = *reinterpret_cast<const lat_bf16x8*>(k1 + 32 * c);
+                }
+                sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[c], sa, 0, 0, 0);
+                sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kc, qf[c], sb, 0, 0, 0);
+            }
+        }
+        // this lane: head `col`, keys kb + 4 g + i (sa) and kb + 16 + 4 g + i (sb)
+        float s[8];
+        float m_new = m_run;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int key = kb + (i < 4 ? 4 * g + i : 16 + 4 * g + i - 4);
+            const float raw = (i < 4 ? sa[i] : sb[i - 4]) * scale;
+            s[i] = key <= pos && !no_page ? raw : -INFINITY;
+            m_new = fmaxf(m_new, s[i]);
+        }
+        m_new = nva_max_over_rows(m_new);
+        const float m_use = fmaxf(m_new, -1e30f);
+        lat_bf16x8 pf;
+        float psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const __bf16 p = (__bf16)__builtin_amdgcn_exp2f((s[i] - m_use) * log2e);
+            pf[i] = p;
+            psum += (float)p;              // the sum of what the product below really uses
+        }
+        psum = nva_sum_over_rows(psum);
+        const float alpha = __builtin_amdgcn_exp2f((fmaxf(m_run, -1e30f) - m_use) * log2e);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        // ---- O^T += V^T P^T: channel 16 b + col, keys kb + 4 g .. + 3 and kb + 16 + 4 g .. + 3
+        const __bf16* v0 = v_cache + (((int64_t)page * tiles_per_page + in_page / LAT_TILE) * rank + col) * LAT_TILE + 4 * g;
+        const bool whole = kb + LAT_TILE - 1 <= pos && !no_page;
+#pragma unroll
+        for (int b = 0; b < CB; ++b) {
+            if (b < blocks) {
+                const lat_bf16x4 lo = *reinterpret_cast<const lat_bf16x4*>(v0 + (int64_t)b * 16 * LAT_TILE);
+                const lat_bf16x4 hi = *reinterpret_cast<const lat_bf16x4*>(v0 + (int64_t)b * 16 * LAT_TILE + 16);
+                lat_bf16x8 vf;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) vf[e] = lo[e], vf[4 + e] = hi[e];
+                if (!whole) {              // what the cache holds beyond the token's own key may be anything
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (no_page || kb + (e < 4 ? 4 * g + e : 16 + 4 * g + e - 4) > pos) vf[e] = (__bf16)0.f;
+                }
+                lat_f32x4 a = acc[b];
+                a[0] *= alpha; a[1] *= alpha; a[2] *= alpha; a[3] *= alpha;
+                acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, a, 0, 0, 0);
+            }
+        }
+    }
+    // acc[b][i] = O[head col][channel 16 b + 4 g + i]
+    if (!head_ok) return;
+    if (shares == 1) {
+        const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+        __bf16* orow = out + t * out_stride + (int64_t)head * rank;
+#pragma unroll
+        for (int b = 0; b < CB; ++b)
+            if (b < blocks) {
+                lat_bf16x4 v;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[i] = (__bf16)(acc[b][i] * inv);
+                *reinterpret_cast<lat_bf16x4*>(orow + 16 * b + 4 * g) = v;
+            }
+        return;
+    }
+    float* mine = part + ((t * heads + head) * shares + share) * (int64_t)(2 + rank);
+    if (g == 0) mine[0] = m_run, mine[1] = l_run;
+#pragma unroll
+    for (int b = 0; b < CB; ++b)
+        if (b < blocks) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) mine[2 + 16 * b + 4 * g + i] = acc[b][i];
+        }
+}
+
+// One wave per (token, head): the shares' results joined, in the order of the shares.
+__global__ void __launch_bounds__(NVA_WAVE)
+latent_attn_merge_kernel(const float* __restrict__ part, int shares, __bf16* __restrict__ out, int64_t out_stride,
+                         int heads, int rank) {
+    const int64_t t = blockIdx.x;
+    const int h = blockIdx.y, lane = threadIdx.x;
+    const float* mine = part + (t * heads + h) * shares * (int64_t)(2 + rank);
+    float m = -INFINITY;
+    for (int s = 0; s < shares; ++s) m = fmaxf(m, mine[s * (int64_t)(2 + rank)]);
+    float l = 0.f;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < shares; ++s) {
+        const float* p = mine + s * (int64_t)(2 + rank);
+        if (p[0] == -INFINITY) continue;
+        const float f = __expf(p[0] - m);
+        l += p[1] * f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int d = lane + i * NVA_WAVE;
+            if (d < rank) acc[i] += p[2 + d] * f;
+        }
+    }
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    __bf16* orow = out + t * out_stride + (int64_t)h * rank;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int d = lane + i * NVA_WAVE;
+        if (d < rank) orow[d] = (__bf16)(acc[i] * inv);
+    }
+}
+
+// q2 [tokens, heads * (rank + rot)], out [tokens, heads * rank]; K cache [pages, 1, page, rank + rot], V cache
+// [pages, 1, page / 32, rank, 32]; part: float [tokens * heads * shares * (2 + rank)] where shares > 1.
+// Returns 1 (and a message) for sizes it does not take: the caller runs the general kernel then.
+NVA_EXPORT int nva_latent_attention_bf16(const void* q2, int64_t q_stride, void* out, int64_t out_stride, float* part,
+                                         int shares, const void* k_cache, const void* v_cache,
+                                         const int32_t* block_tables, int table_stride, const int32_t* token_seq,
+                                         const int32_t* positions, int64_t tokens, int heads, int rank, int rot,
+                                         int page_size, float scale, const float* sinks, int32_t* error_flag,
+                                         hipStream_t stream) {
+    if (tokens == 0) return 0;
+    if (rank % 16 || rank <= 0 || rank > 512 || rot % 8 || rot <= 0 || rot > LAT_MAX_ROT || page_size % LAT_TILE || page_size <= 0) {
+        nva_fail("latent_attention: needs a latent of a multiple of 16 up to 512, a rotated part of a multiple of 8 up to %d and "
+                 "pages of a multiple of %d keys (got %d, %d, %d)", LAT_MAX_ROT, LAT_TILE, rank, rot, page_size);
+        return 1;
+    }
+    if (tokens < 0 || tokens > 0x7fffffff || heads <= 0 || shares < 1 || shares > 65535 || (shares > 1 && !part) ||
+        table_stride <= 0 || !(scale > 0.f))
+        return nva_fail("latent_attention: bad sizes tokens=%lld heads=%d shares=%d", (long long)tokens, heads, shares);
+    if (q_stride % 8 || out_stride % 4 || !nva_aligned(q2, 16) || !nva_aligned(out, 8) || !nva_aligned(k_cache, 16) ||
+        !nva_aligned(v_cache, 8)) {
+        nva_fail("latent_attention: rows that are not aligned for vector access");
+        return 1;
+    }
+    dim3 grid((unsigned)tokens, (unsigned)shares, (unsigned)((heads + 15) / 16));
+#define LAT_LAUNCH(MC)                                                                                               \
+    hipLaunchKernelGGL(latent_attn_kernel<MC>, grid, dim3(NVA_WAVE), 0, stream, (const __bf16*)q2, q_stride,            \
+                       (__bf16*)out, out_stride, part, (const __bf16*)k_cache, (const __bf16*)v_cache, block_tables,     \
+                       table_stride, token_seq, positions, heads, rank, rot, page_size, scale, sinks, error_flag)
+    if (rank <= 128) LAT_LAUNCH(128);
+    else if (rank <= 256) LAT_LAUNCH(256);
+    else if (rank <= 384) LAT_LAUNCH(384);
+    else LAT_LAUNCH(512);
+#undef LAT_LAUNCH
+    if (shares > 1)
+        hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)tokens, (unsigned)heads), dim3(NVA_WAVE), 0, stream, part,
+                           shares, (__bf16*)out, out_stride, heads, rank);
+    return nva_check_launch("latent_attention");
+}
+#endif
+
 NVA_DEFINE_LAST_ERROR(nva_latent)

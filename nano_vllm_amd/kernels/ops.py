@@ -1374,13 +1374,12 @@ class HipKernels:
         if sigmoid_bias is not None and (sigmoid_bias.dtype != torch.float32 or sigmoid_bias.shape != (num_heads,) or
                                          not sigmoid_bias.is_contiguous() or sinks is not None):
             raise KernelError(f"attention: sigmoid_bias must be contiguous float32 [{num_heads}] and goes without sinks")
-        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and v_dim == head_dim \
-            and sigmoid_bias is None
+        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and v_dim == head_dim
         if batch.num_decode > 0 and mfma and \
                 self._decode_kernel_takes(num_heads // num_kv_heads, head_dim, page_size, q, qs, out, os_):
             start = batch.num_decode
             self._attention_decode(q, qs, out, os_, k_cache, v_cache, tables, batch, start, num_heads, num_kv_heads,
-                                   head_dim, page_size, scale, window, sinks, chunk, keep, cap)
+                                   head_dim, page_size, scale, window, sinks, chunk, keep, cap, sigmoid_bias)
         if batch.num_decode < tokens and mfma and \
                 self._prefill_kernel_takes(head_dim, page_size, tables.shape[1], q, qs, out, os_):
             # portions of prompts: the matrix-core prefill kernel, one workgroup per 32 query rows
@@ -1389,7 +1388,8 @@ class HipKernels:
                          _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.cu_seqlens_q), _p(batch.kv_lens),
                          _p(tiles), c_i64(tiles.shape[0]), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
-                         c_i32(chunk or 0), c_i32(keep), c_f32(cap), _p(sinks), _p(self.fault_flag), self._stream())
+                         c_i32(chunk or 0), c_i32(keep), c_f32(cap), _p(sinks), _p(sigmoid_bias), _p(self.fault_flag),
+                         self._stream())
             tokens = batch.num_decode            # what is left: the single tokens before the portions, if any
         if self.tiled_general_attention and start <= batch.num_decode < tokens and not window and sigmoid_bias is None and \
                 max(head_dim, v_dim) <= GENERAL_TILED_MAX_HEAD_DIM:
@@ -1447,6 +1447,43 @@ class HipKernels:
                      c_i32(dim), c_i32(rot), c_i32(rank), _p(weight), c_i32(wf), c_f32(eps), _p(rot_table), _p(q2),
                      c_i64(q2.shape[1]), _p(slots), _p(k_cache), _p(v_cache), c_i32(page_size), self._stream())
         return q2
+
+    def latent_attention(self, q2: torch.Tensor, heads: int, rank: int, rot: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                         batch, group: int, scale: float, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Causal softmax attention of heads that share one key/value head whose key rows are [latent | rotated part]
+        (rank + rot entries) and whose value rows are the latent: q2 [tokens, heads * (rank + rot)] -> [tokens, heads *
+        rank].  bfloat16 with a latent of a multiple of 16 runs on the matrix cores (a token's heads are the columns of
+        the products, so a key row is fetched once for all of them; a token's keys are shared out among workgroups
+        where a step has few tokens); everything else runs the general attention kernel."""
+        q2 = _t(q2)
+        tokens, width, qs = _rows2d(q2, "latent attention q")
+        page_size = self._check_cache(k_cache, v_cache, 1, rank + rot, q2.dtype, rank)
+        if self.mfma_attention and q2.dtype == torch.bfloat16 and rank % 16 == 0 and 0 < rank <= 512 and rot % 8 == 0 and \
+                0 < rot <= 128 and page_size % 32 == 0 and qs % 8 == 0 and 0.0 < scale < float("inf"):
+            if width != heads * (rank + rot):
+                raise KernelError("latent attention: q width is not heads * (rank + rot)")
+            if sinks is not None and (sinks.dtype != torch.float32 or sinks.shape != (heads,) or not sinks.is_contiguous()):
+                raise KernelError(f"latent attention: sinks must be contiguous float32 [{heads}]")
+            tables = batch.groups[group].block_tables
+            if tables.dtype != torch.int32 or tables.dim() != 2 or tables.shape[0] != batch.num_seqs or not tables.is_contiguous():
+                raise KernelError("latent attention: block tables must be contiguous int32 [requests, pages]")
+            if tables.shape[1] < (batch.max_kv_len + page_size - 1) // page_size:
+                raise KernelError("latent attention: the block tables are too narrow for the step's longest request")
+            _i32(batch.token_seq, tokens, "token_seq")
+            _i32(batch.positions, tokens, "positions")
+            out = torch.empty((tokens, heads * rank), dtype=q2.dtype, device=q2.device)
+            # few tokens with many keys: a token's tiles of 32 keys are shared out, four tiles a share or more, until
+            # about two waves a compute unit run; the number follows from the step's shape alone
+            blocks = (heads + 15) // 16
+            shares = max(1, min(64, ((batch.max_kv_len + 31) // 32) // 4, 512 // (tokens * blocks)))
+            part = torch.empty(tokens * heads * shares * (2 + rank), dtype=torch.float32, device=q2.device) if shares > 1 else None
+            library.call("latent", "bf16", "nva_latent_attention", _p(q2), c_i64(qs), _p(out), c_i64(out.shape[1]), _p(part),
+                         c_i32(shares), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.token_seq),
+                         _p(batch.positions), c_i64(tokens), c_i32(heads), c_i32(rank), c_i32(rot), c_i32(page_size),
+                         c_f32(scale), _p(sinks), _p(self.fault_flag), self._stream())
+            return out
+        return self.paged_attention(q2, heads, 1, rank + rot, k_cache, v_cache, batch, group, scale, None, v_head_dim=rank,
+                                    sinks=sinks)
 
     def heads_linear(self, x: torch.Tensor, x_head: int, w: torch.Tensor, heads: int, n_out: int, k_in: int,
                      transposed: bool, y: torch.Tensor, y_head: int, y_offset: int = 0) -> torch.Tensor:
@@ -1729,7 +1766,7 @@ class HipKernels:
                                                                              out_stride)
 
     def _attention_decode(self, q, qs, out, os_, k_cache, v_cache, tables, batch, n, num_heads, num_kv_heads,
-                          head_dim, page_size, scale, window, sinks=None, chunk=None, keep=0, cap=0.0):
+                          head_dim, page_size, scale, window, sinks=None, chunk=None, keep=0, cap=0.0, sigmoid_bias=None):
         # The work is shared out on the device from the tokens' positions, once per step and (kv
         # heads, window): the first layer that asks makes the plan, the others find it on the batch.
         # The library says how large the partial results may get for this many tokens of at most
@@ -1757,7 +1794,7 @@ class HipKernels:
                          _p(scratch), _p(plan), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
                          c_i64(t1 - t0), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_f32(cap),
-                         c_i32(bound), c_i32(waves), _p(sinks), _p(self.fault_flag), self._stream())
+                         c_i32(bound), c_i32(waves), _p(sinks), _p(sigmoid_bias), _p(self.fault_flag), self._stream())
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:

@@ -1,7 +1,7 @@
 """Named config.json contents for runs with random weights (there is no checkpoint to read
 them from): two tiny test shapes and the Qwen3 dense sizes that the benchmarks use, three
 Nozurax shapes (a tiny one, and layers of the Qwen3 1.7B and 8B sizes), two Mafarax shapes (a tiny
-one, and layers of the Qwen3 1.7B sizes) and two Kirisun shapes of the same kind.  These are
+one, and layers of the Qwen3 1.7B sizes) and two Kirisun and two Pemuvik shapes of the same kind.  These are
 inputs, as a model folder's config.json is; nothing in the model code reads them.
 
     python -m nano_vllm_amd.cli random-model --shape qwen3-8b --config-only --out DIR
@@ -80,7 +80,39 @@ def _kirisun(layers, width, heads, kv_heads, dim, vdim, inner, vocab, window, ke
             "torch_dtype": dtype}
 
 
+def _pemuvik(layers, width, heads, kv_heads, dim, vdim, inner, vocab, window, eps=1e-6, dtype="bfloat16", rot=None,
+             latent_heads=None, latent_dim=None, latent_rot=None, latent_vdim=None, kv_rank=None, experts=32, top=8, identity=2,
+             group_count=1, group_keep=1, pattern=(("attention", "moe"), ("latent_attention", "dense"))) -> dict:
+    """Layers that follow `pattern` in turn: the window attention with sigmoid weights (half the head rotated, values
+    normed and mixed with the first such layer's) and the attention through a latent (as many heads as the other has
+    query heads, a latent of kv_rank entries and a rotated key part of half a head unless named), each with a dense
+    gated layer of `inner` or with `top` of `experts` gated experts of inner / top each (and `identity` outputs that
+    give the input back) beside a shared expert of inner / 4."""
+    lh, ld, lv = latent_heads or heads, latent_dim or dim, latent_vdim or vdim
+    lr = latent_rot or max(2, dim // 2)
+    mixers = {
+        "attention": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "v_mix": True,
+                      "mask": {"size": window}, "rot": {"dims": rot or dim // 2, "base": 1e6}},
+        "latent_attention": {"heads": lh, "dim": ld, "rot_dim": lr, "vdim": lv, "kv_rank": kv_rank or 3 * dim,
+                             "scale": (ld + lr) ** -0.5, "rot": {"dims": lr, "base": 1e4}},
+    }
+    mlps = {
+        "dense": {"kind": "dense", "ff": inner},
+        "moe": {"kind": "moe", "expert": {"ff": max(1, inner // top)}, "shared": {"ff": max(1, inner // 4)},
+                "router": {"experts": experts, "top": top, "identity": identity,
+                           "groups": {"count": group_count, "keep": group_keep}}},
+        None: None,
+    }
+    return {"architecture": "Pemuvik", "vocab": vocab, "width": width, "norm": {"eps": eps},
+            "layers": [{"type": pattern[i % len(pattern)][0], "mixer": mixers[pattern[i % len(pattern)][0]],
+                        "mlp": mlps[pattern[i % len(pattern)][1]]} for i in range(layers)],
+            "torch_dtype": dtype}
+
+
 SHAPES: Dict[str, dict] = {
+    "pemuvik-tiny": _pemuvik(4, 64, 4, 2, 16, 24, 96, 256, window=12, eps=1e-5, dtype="float32", rot=8, latent_heads=2, latent_dim=12,
+                             latent_rot=4, latent_vdim=8, kv_rank=20, experts=6, top=2, identity=2, group_count=4, group_keep=2),
+    "pemuvik-1b": _pemuvik(16, 2048, 16, 8, 128, 128, 6144, 32768, window=1024, experts=30, group_count=4, group_keep=2),
     "kirisun-tiny": _kirisun(4, 64, 4, 2, 16, 24, 96, 256, window=12, keep_first=3, eps=1e-5, dtype="float32", rot=8, softcap=5.0,
                              delta_heads=4, delta_kv_heads=2, delta_dim=12, delta_vdim=8, conv=3, rank=3, experts=6, top=2),
     "kirisun-1b": _kirisun(16, 2048, 16, 8, 128, 128, 6144, 32768, window=1024),

@@ -147,7 +147,7 @@ class Attention(Part):
     def kernel_modules(self):
         prepare = "qk_rownorm" if self.row_prepare else "rope"
         rope = ("rope",) if self.row_prepare and self.position_encoding else ()
-        if self.v_head_dim != self.head_dim or self.weighting == "sigmoid":
+        if self.v_head_dim != self.head_dim:
             return (prepare, "attn_generic") + rope
         return (prepare, "attn_generic", "attn_decode", "attn_prefill") + \
             (("rope",) if self.row_prepare and self.position_encoding else ())

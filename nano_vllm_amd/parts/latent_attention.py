@@ -12,7 +12,7 @@ latent row per token, which is all that is cached.
 
 Since q_plain . (Wuk_h c) = (Wuk_h^T q_plain) . c, neither keys nor values are ever formed: the cache holds one key
 row [c | kr] and one value row c per token (one key/value head of C + R and C entries), a head's query becomes
-[Wuk_h^T q_plain | q_turned], the engine's paged attention runs on that, and Wuv_h is applied to its output.
+[Wuk_h^T q_plain | q_turned], the attention runs on that (kernels.latent_attention), and Wuv_h is applied to its output.
 The two small products per head are kernels.heads_linear.
 """
 from __future__ import annotations
@@ -89,8 +89,7 @@ class LatentAttention(Part):
                               group.slot_mapping, cache.k, cache.v)
         # the plain parts of the queries into the latent's space: q2[t, h, :C] = Wuk_h^T q[t, h, :D]
         k.heads_linear(proj, D + R, w[f"{self.uk_name}.weight"], H, C, D, True, q2, C + R)
-        o = k.paged_attention(q2, H, 1, C + R, cache.k, cache.v, batch, cache.group, self.scale, None, v_head_dim=C,
-                              sinks=w.get("sinks"))
+        o = k.latent_attention(q2, H, C, R, cache.k, cache.v, batch, cache.group, self.scale, sinks=w.get("sinks"))
         # and the outputs out of it: heads[t, h, :V] = Wuv_h o[t, h, :C]
         heads = o.new_empty((o.shape[0], H * V))
         k.heads_linear(o, C, w[f"{self.uv_name}.weight"], H, V, C, False, heads, V)

@@ -87,14 +87,15 @@ def window_values(h, m, w, p, eps, shared):
     return v
 
 
-def sigmoid_window_attend(q, k, v, m, bias):
-    """q [T, H, D], k [T, G, D], v [T, G, DV] -> [T, H * DV]: every visible key weighs sigmoid(score + bias)."""
+def sigmoid_window_attend(q, k, v, m, bias, rows=None):
+    """q [T, H, D], k [T, G, D], v [T, G, DV] -> [T, H * DV]: every visible key weighs sigmoid(score + bias).
+    rows: the tokens whose output is wanted (default all; the others' stay zero)."""
     T, H = q.shape[0], q.shape[1]
     per = H // k.shape[1]
     out = torch.zeros(T, H, v.shape[2], dtype=q.dtype)
     for head in range(H):
         g = head // per
-        for i in range(T):
+        for i in (range(T) if rows is None else rows):
             for j in range(max(0, i - m["mask"]["size"] + 1) if m.get("mask") else 0, i + 1):
                 weight = torch.sigmoid(torch.dot(q[i, head], k[j, g]) * m["scale"] + bias[head])
                 out[i, head] += weight * v[j, g]

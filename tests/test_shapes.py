@@ -10,7 +10,7 @@ def test_named_shapes_are_valid_configurations():
     for name in SHAPES:
         cj = shape(name)
         cfg = architecture_of(cj).parse_config(cj)
-        if name.split("-")[0] in ("nozurax", "mafarax", "kirisun"):
+        if name.split("-")[0] in ("nozurax", "mafarax", "kirisun", "pemuvik"):
             assert cfg.to_dict()["width"] == cj["width"] and len(cfg.layers) == len(cj["layers"])
             assert architecture_of(cfg.to_dict()).parse_config(cfg.to_dict()) == cfg
             continue

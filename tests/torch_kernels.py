@@ -568,6 +568,10 @@ class TorchKernels:
             v_cache[page, 0, off // vt, :, off % vt] = c[ok]
         return q2.reshape(T, heads * (rank + rot))
 
+    def latent_attention(self, q2, heads, rank, rot, k_cache, v_cache, batch, group, scale, sinks=None):
+        return self.paged_attention(q2, heads, 1, rank + rot, k_cache, v_cache, batch, group, scale, None, v_head_dim=rank,
+                                    sinks=sinks)
+
     def heads_linear(self, x, x_head, w, heads, n_out, k_in, transposed, y, y_head, y_offset=0):
         wh = w.float().reshape(heads, k_in, n_out).transpose(1, 2) if transposed else w.float().reshape(heads, n_out, k_in)
         for h in range(heads):
