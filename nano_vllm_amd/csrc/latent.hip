@@ -155,6 +155,75 @@ NVA_EXPORT int NVA_NAME(nva_heads_linear)(const void* x, int64_t x_stride, int64
 }
 
 #if defined(NVA_BF16)
+// ---------------------------------------------------------------------------- the product per head on the matrix cores
+// W [heads, n_out, k_in] with k side by side.  A wave takes 16 tokens of one head and 64 outputs: the rows of W are the
+// A operand and the tokens' rows the B operand of v_mfma_f32_16x16x32_bf16, both straight from global memory (a lane 16
+// bytes a load); a fragment of x serves four products.  The sum over k runs in the order of the steps of 32, whatever
+// the other tokens of the tile.
+typedef __attribute__((ext_vector_type(8))) __bf16 hl_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float hl_f32x4;
+
+__global__ void __launch_bounds__(NVA_WAVE)
+heads_linear_mfma_kernel(const __bf16* __restrict__ x, int64_t x_stride, int64_t x_head, const __bf16* __restrict__ w,
+                         __bf16* __restrict__ y, int64_t y_stride, int64_t y_head, int64_t tokens, int n_out, int k_in) {
+    const int64_t t0 = (int64_t)blockIdx.x * 16;
+    const int h = blockIdx.y, n0 = blockIdx.z * 64;
+    const int lane = threadIdx.x, col = lane & 15, g = lane >> 4;
+    const int64_t t = t0 + col;
+    const __bf16* xr = x + (t < tokens ? t : tokens - 1) * x_stride + h * x_head + 8 * g;
+    const __bf16* wr[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) wr[b] = w + ((int64_t)h * n_out + min(n0 + 16 * b + col, n_out - 1)) * k_in + 8 * g;
+    hl_f32x4 acc[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) acc[b] = hl_f32x4{0.f, 0.f, 0.f, 0.f};
+    const int k_last = k_in - 8;                    // k_in is a multiple of 8: a piece lies inside the row or outside
+#pragma unroll 4
+    for (int k0 = 0; k0 < k_in; k0 += 32) {
+        const bool inside = k0 + 8 * g <= k_last;
+        const int at = inside ? k0 : -8 * g;        // (every load unconditional: a piece outside the row reads the row's first, and counts as zero)
+        hl_bf16x8 xf = *reinterpret_cast<const hl_bf16x8*>(xr + at);
+        hl_bf16x8 wf[4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) wf[b] = *reinterpret_cast<const hl_bf16x8*>(wr[b] + at);
+        if (!inside) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) xf[e] = (__bf16)0.f;
+        }
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[b], xf, acc[b], 0, 0, 0);
+    }
+    // acc[b][i] = y[token col][n0 + 16 b + 4 g + i]
+    if (t >= tokens) return;
+    __bf16* yr = y + t * y_stride + h * y_head;
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int n = n0 + 16 * b + 4 * g + i;
+            if (n < n_out) yr[n] = (__bf16)acc[b][i];
+        }
+}
+
+// As nva_heads_linear with w_n = k_in, w_k = 1 (W [heads * n_out, k_in], contiguous).  Returns 1 (and a message) for
+// shapes it does not take: k_in a multiple of 8, x rows and heads at multiples of 8 elements, 16-byte aligned pointers.
+NVA_EXPORT int nva_heads_linear_mfma_bf16(const void* x, int64_t x_stride, int64_t x_head, const void* w, void* y,
+                                          int64_t y_stride, int64_t y_head, int64_t tokens, int heads, int n_out, int k_in,
+                                          hipStream_t stream) {
+    if (tokens == 0) return 0;
+    if (k_in % 8 || k_in <= 0 || x_stride % 8 || x_head % 8 || !nva_aligned(x, 16) || !nva_aligned(w, 16)) {
+        nva_fail("heads_linear_mfma: rows that are not aligned for 16-byte loads (k_in %d)", k_in);
+        return 1;
+    }
+    if (tokens < 0 || tokens > 0x7fffffffLL * 16 || heads <= 0 || heads > 65535 || n_out <= 0 || (n_out + 63) / 64 > 65535 ||
+        !x || !w || !y)
+        return nva_fail("heads_linear_mfma: bad sizes tokens=%lld heads=%d outputs=%d", (long long)tokens, heads, n_out);
+    dim3 grid((unsigned)((tokens + 15) / 16), (unsigned)heads, (unsigned)((n_out + 63) / 64));
+    hipLaunchKernelGGL(heads_linear_mfma_kernel, grid, dim3(NVA_WAVE), 0, stream, (const __bf16*)x, x_stride, x_head,
+                       (const __bf16*)w, (__bf16*)y, y_stride, y_head, tokens, n_out, k_in);
+    return nva_check_launch("heads_linear_mfma");
+}
+
 // ---------------------------------------------------------------------------- the attention itself, on the matrix cores
 // One key/value head for all query heads: the query heads of a token are the 16 columns of the products, so a key row
 // that is fetched serves all of them.  A wave takes one token, 16 of its heads and a share of its keys, in tiles of 32:
@@ -223,19 +292,32 @@ latent_attn_kernel(const __bf16* __restrict__ q2, int64_t q_stride, __bf16* __re
         // ---- scores: rows of K as they lie, keys kb + col and kb + 16 + col
         const __bf16* k0 = k_cache + ((int64_t)page * page_size + in_page + col) * width + 8 * g;
         const __bf16* k1 = k0 + (int64_t)16 * width;
+        // (all of the tile's loads are asked for before anything is used: a wave is alone on its SIMD, and what it has
+        // on its way is all that hides the memory's latency)
+        const __bf16* v0 = v_cache + (((int64_t)page * tiles_per_page + in_page / LAT_TILE) * rank + col) * LAT_TILE + 4 * g;
+        lat_bf16x8 ka[KS], kc[KS];
+        lat_bf16x4 vlo[CB], vhi[CB];
+#pragma unroll
+        for (int c = 0; c < KS; ++c) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ka[c][e] = kc[c][e] = (__bf16)0.f;
+            if (c < steps && 32 * c + 8 * g < width) {
+                ka[c] = *reinterpret_cast<const lat_bf16x8*>(k0 + 32 * c);
+                kc[c] = *reinterpret_cast<const lat_bf16x8*>(k1 + 32 * c);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < CB; ++b)
+            if (b < blocks) {
+                vlo[b] = *reinterpret_cast<const lat_bf16x4*>(v0 + (int64_t)b * 16 * LAT_TILE);
+                vhi[b] = *reinterpret_cast<const lat_bf16x4*>(v0 + (int64_t)b * 16 * LAT_TILE + 16);
+            }
         lat_f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int c = 0; c < KS; ++c) {
             if (c < steps) {
-                lat_bf16x8 ka, kc;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) ka[e] = kc[e] = (__bf16)0.f;
-                if (32 * c + 8 * g < width) {
-                    ka = *reinterpret_cast<const lat_bf16x8*>(k0 + 32 * c);
-                    kc = *reinterpret_cast<const lat_bf16x8*>(k1 + 32 * c);
-                }
-                sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[c], sa, 0, 0, 0);
-                sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kc, qf[c], sb, 0, 0, 0);
+                sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c], qf[c], sa, 0, 0, 0);
+                sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kc[c], qf[c], sb, 0, 0, 0);
             }
         }
         // this lane: head `col`, keys kb + 4 g + i (sa) and kb + 16 + 4 g + i (sb)
@@ -263,16 +345,13 @@ latent_attn_kernel(const __bf16* __restrict__ q2, int64_t q_stride, __bf16* __re
         l_run = l_run * alpha + psum;
         m_run = m_new;
         // ---- O^T += V^T P^T: channel 16 b + col, keys kb + 4 g .. + 3 and kb + 16 + 4 g .. + 3
-        const __bf16* v0 = v_cache + (((int64_t)page * tiles_per_page + in_page / LAT_TILE) * rank + col) * LAT_TILE + 4 * g;
         const bool whole = kb + LAT_TILE - 1 <= pos && !no_page;
 #pragma unroll
         for (int b = 0; b < CB; ++b) {
             if (b < blocks) {
-                const lat_bf16x4 lo = *reinterpret_cast<const lat_bf16x4*>(v0 + (int64_t)b * 16 * LAT_TILE);
-                const lat_bf16x4 hi = *reinterpret_cast<const lat_bf16x4*>(v0 + (int64_t)b * 16 * LAT_TILE + 16);
                 lat_bf16x8 vf;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) vf[e] = lo[e], vf[4 + e] = hi[e];
+                for (int e = 0; e < 4; ++e) vf[e] = vlo[b][e], vf[4 + e] = vhi[b][e];
                 if (!whole) {              // what the cache holds beyond the token's own key may be anything
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
@@ -309,7 +388,7 @@ latent_attn_kernel(const __bf16* __restrict__ q2, int64_t q_stride, __bf16* __re
         }
 }
 
-// One wave per (token, head): the shares' results joined, in the order of the shares.
+// One wave per (token, head, 128 channels): the shares' results joined, in the order of the shares.
 __global__ void __launch_bounds__(NVA_WAVE)
 latent_attn_merge_kernel(const float* __restrict__ part, int shares, __bf16* __restrict__ out, int64_t out_stride,
                          int heads, int rank) {
@@ -319,23 +398,32 @@ latent_attn_merge_kernel(const float* __restrict__ part, int shares, __bf16* __r
     float m = -INFINITY;
     for (int s = 0; s < shares; ++s) m = fmaxf(m, mine[s * (int64_t)(2 + rank)]);
     float l = 0.f;
-    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < shares; ++s) {
-        const float* p = mine + s * (int64_t)(2 + rank);
-        if (p[0] == -INFINITY) continue;
-        const float f = __expf(p[0] - m);
-        l += p[1] * f;
+    float acc[2] = {0.f, 0.f};
+    const int d0 = blockIdx.z * 2 * NVA_WAVE + lane;                 // this lane's channels: d0 and d0 + 64
+    // (four shares at a time, their loads unconditional: a share without keys has weight zero)
+    for (int s0 = 0; s0 < shares; s0 += 4) {
+        float f[4], ls[4], v[4][2];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int d = lane + i * NVA_WAVE;
-            if (d < rank) acc[i] += p[2 + d] * f;
+        for (int j = 0; j < 4; ++j) {
+            const float* p = mine + min(s0 + j, shares - 1) * (int64_t)(2 + rank);
+            const float ms = p[0];
+            ls[j] = p[1];
+            f[j] = (s0 + j >= shares || ms == -INFINITY) ? 0.f : __expf(ms - m);
+#pragma unroll
+            for (int i = 0; i < 2; ++i) v[j][i] = d0 + i * NVA_WAVE < rank ? p[2 + d0 + i * NVA_WAVE] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            l += ls[j] * f[j];
+            acc[0] += v[j][0] * f[j];
+            acc[1] += v[j][1] * f[j];
         }
     }
     const float inv = l > 0.f ? 1.f / l : 0.f;
     __bf16* orow = out + t * out_stride + (int64_t)h * rank;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int d = lane + i * NVA_WAVE;
+    for (int i = 0; i < 2; ++i) {
+        const int d = d0 + i * NVA_WAVE;
         if (d < rank) orow[d] = (__bf16)(acc[i] * inv);
     }
 }
@@ -374,7 +462,8 @@ NVA_EXPORT int nva_latent_attention_bf16(const void* q2, int64_t q_stride, void*
     else LAT_LAUNCH(512);
 #undef LAT_LAUNCH
     if (shares > 1)
-        hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)tokens, (unsigned)heads), dim3(NVA_WAVE), 0, stream, part,
+        hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)tokens, (unsigned)heads, (unsigned)((rank + 127) / 128)),
+                           dim3(NVA_WAVE), 0, stream, part,
                            shares, (__bf16*)out, out_stride, heads, rank);
     return nva_check_launch("latent_attention");
 }

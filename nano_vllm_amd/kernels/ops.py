@@ -1489,7 +1489,8 @@ class HipKernels:
                      transposed: bool, y: torch.Tensor, y_head: int, y_offset: int = 0) -> torch.Tensor:
         """A product per head: y[t, h * y_head + y_offset + n] = sum_k W[h][n][k] x[t, h * x_head + k], n < n_out, k < k_in.
         w is contiguous [heads * n_out, k_in], or with transposed [heads * k_in, n_out] (W[h][n][k] = w[h * k_in + k, n]).
-        x and y are 2-d with rows of any stride.  Float sums over k in ascending order, rounded once."""
+        x and y are 2-d with rows of any stride.  Float sums over k in ascending order, rounded once (bfloat16 with
+        matrices that are not transposed: on the matrix cores, in the order of their steps of 32)."""
         x = _t(x)
         tokens, xw, xs = _rows2d(x, "heads_linear input")
         yrows, yw, ys = _rows2d(y, "heads_linear output")
@@ -1500,6 +1501,11 @@ class HipKernels:
             raise KernelError("heads_linear: the heads do not fit the rows")
         w_n, w_k = (1, n_out) if transposed else (k_in, 1)
         yv = y[:, y_offset:] if y_offset else y
+        if x.dtype == torch.bfloat16 and not transposed and k_in % 8 == 0 and xs % 8 == 0 and x_head % 8 == 0 and \
+                x.data_ptr() % 16 == 0 and self.mfma_attention:
+            library.call("latent", "bf16", "nva_heads_linear_mfma", _p(x), c_i64(xs), c_i64(x_head), _p(w), _p(yv), c_i64(ys),
+                         c_i64(y_head), c_i64(tokens), c_i32(heads), c_i32(n_out), c_i32(k_in), self._stream())
+            return y
         library.call("latent", _suffix(x), "nva_heads_linear", _p(x), c_i64(xs), c_i64(x_head), _p(w), c_i64(n_out * k_in),
                      c_i64(w_n), c_i64(w_k), _p(yv), c_i64(ys), c_i64(y_head), c_i64(tokens), c_i32(heads), c_i32(n_out),
                      c_i32(k_in), self._stream())

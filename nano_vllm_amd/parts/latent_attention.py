@@ -80,6 +80,12 @@ class LatentAttention(Part):
     def cache_need(self):
         return PagedKV(1, self.rank + self.rot, None, self.rank)
 
+    def on_weights_loaded(self) -> None:
+        # Wuk_h^T, one below the other: [heads * rank, head_dim], the rows of the product that takes the queries' plain
+        # parts into the latent's space (made once; the checkpoint's own layout serves the keys, which are never formed)
+        uk = self.weights[f"{self.uk_name}.weight"]
+        self._uk_t = uk.view(self.heads, self.dim, self.rank).transpose(1, 2).contiguous().view(self.heads * self.rank, self.dim)
+
     def forward(self, x, batch, cache):
         k, w = self.kernels, self.weights
         H, D, R, C, V = self.heads, self.dim, self.rot, self.rank, self.vdim
@@ -88,7 +94,7 @@ class LatentAttention(Part):
         q2 = k.latent_prepare(proj, H, D, R, C, w["c_norm.weight"], self.eps, self.position_encoding.step_table(batch),
                               group.slot_mapping, cache.k, cache.v)
         # the plain parts of the queries into the latent's space: q2[t, h, :C] = Wuk_h^T q[t, h, :D]
-        k.heads_linear(proj, D + R, w[f"{self.uk_name}.weight"], H, C, D, True, q2, C + R)
+        k.heads_linear(proj, D + R, self._uk_t, H, C, D, False, q2, C + R)
         o = k.latent_attention(q2, H, C, R, cache.k, cache.v, batch, cache.group, self.scale, sinks=w.get("sinks"))
         # and the outputs out of it: heads[t, h, :V] = Wuv_h o[t, h, :C]
         heads = o.new_empty((o.shape[0], H * V))
