@@ -251,7 +251,9 @@ latent_attn_kernel(const __bf16* __restrict__ q2, int64_t q_stride, __bf16* __re
                    const float* __restrict__ sinks, int32_t* error_flag) {
     constexpr int KS = (MAXC + LAT_MAX_ROT) / 32;      // steps of 32 channels of the first product, at most
     constexpr int CB = MAXC / 16;                      // blocks of 16 latent channels of the output, at most
-    const int64_t t = blockIdx.x;
+    // (the step's last tokens first: in a prompt's portion they have the most keys, and the workgroups that start first
+    // should be the long ones)
+    const int64_t t = (int64_t)gridDim.x - 1 - blockIdx.x;
     const int share = blockIdx.y, shares = gridDim.y;
     const int lane = threadIdx.x, col = lane & 15, g = lane >> 4;
     const int head = blockIdx.z * 16 + col;
@@ -388,6 +390,185 @@ latent_attn_kernel(const __bf16* __restrict__ q2, int64_t q_stride, __bf16* __re
         }
 }
 
+// The same attention for portions of prompts: a workgroup of four waves takes four tokens in a row of one request (a
+// quarter of an eighth of a row tile of 32 queries; tiles as for the other prefill kernels, most keys first), a wave one
+// token.  The tiles of keys and of transposed values, which the four tokens share, go through LDS once for all of them:
+// the next tile is asked for (into registers) before the products of the tile at hand and stored after them.  The
+// arithmetic of a token is that of latent_attn_kernel with one share, operation for operation.
+template <int MAXC>
+__global__ void __launch_bounds__(4 * NVA_WAVE)
+latent_attn_quad_kernel(const __bf16* __restrict__ q2, int64_t q_stride, __bf16* __restrict__ out, int64_t out_stride,
+                        const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
+                        const int32_t* __restrict__ block_tables, int table_stride, const int32_t* __restrict__ cu_seqlens_q,
+                        const int32_t* __restrict__ kv_lens, const int32_t* __restrict__ row_tiles, int heads, int rank, int rot,
+                        int page_size, float scale, const float* __restrict__ sinks, int32_t* error_flag) {
+    constexpr int KS = (MAXC + LAT_MAX_ROT) / 32, CB = MAXC / 16;
+    constexpr int KP = (MAXC + LAT_MAX_ROT) / 64, VP = MAXC / 64;       // 16-byte pieces of a tile a thread moves, at most
+    extern __shared__ __attribute__((aligned(16))) __bf16 lat_s[];
+    const int width = rank + rot, KSTR = width + 8, VSTR = LAT_TILE + 4;
+    __bf16* const k_s = lat_s;                          // [32 keys][KSTR]
+    __bf16* const v_s = lat_s + LAT_TILE * KSTR;        // [rank channels][VSTR]
+    const int ti = blockIdx.x / 8, quad = blockIdx.x % 8;
+    const int seq = row_tiles[2 * ti], row_tile = row_tiles[2 * ti + 1];
+    const int q_begin = cu_seqlens_q[seq];
+    const int q_len = cu_seqlens_q[seq + 1] - q_begin;
+    const int start = kv_lens[seq] - q_len;             // position of the request's first query of this step
+    const int row0 = row_tile * 32 + quad * 4;
+    if (row0 >= q_len) return;                          // (the whole workgroup)
+    const int tid = threadIdx.x, wave = tid / NVA_WAVE, lane = tid % NVA_WAVE, col = lane & 15, g = lane >> 4;
+    const int row = row0 + wave;
+    const bool token_ok = row < q_len;
+    const int pos = token_ok ? start + row : -1;
+    const int64_t t = q_begin + (token_ok ? row : row0);
+    const int tiles = (start + min(row0 + 3, q_len - 1)) / LAT_TILE + 1;
+    const int head = blockIdx.z * 16 + col;
+    const bool head_ok = head < heads;
+    const int steps = (width + 31) / 32, blocks = rank / 16;
+    const int32_t* table = block_tables + (int64_t)seq * table_stride;
+    const int tiles_per_page = page_size / LAT_TILE;
+    const int k_pieces = 4 * width, v_pieces = 4 * rank;
+
+    lat_bf16x8 qf[KS];
+    const __bf16* qrow = q2 + t * q_stride + (int64_t)(head_ok ? head : 0) * width;
+#pragma unroll
+    for (int c = 0; c < KS; ++c) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[c][e] = (__bf16)0.f;
+        if (c < steps && head_ok && token_ok && 32 * c + 8 * g < width) qf[c] = *reinterpret_cast<const lat_bf16x8*>(qrow + 32 * c + 8 * g);
+    }
+    lat_f32x4 acc[CB];
+#pragma unroll
+    for (int b = 0; b < CB; ++b) acc[b] = lat_f32x4{0.f, 0.f, 0.f, 0.f};
+    const bool with_sink = sinks && head_ok;
+    float m_run = with_sink ? sinks[head] : -INFINITY, l_run = with_sink ? 1.f : 0.f;
+    const float log2e = 1.4426950408889634f;
+
+    lat_bf16x8 kreg[KP], vreg[VP];
+    bool no_page = false, no_page_next = false;
+    auto ask = [&](int tile) __attribute__((always_inline)) {       // a tile's keys and values, as they lie in the cache, into registers
+        const int kb = tile * LAT_TILE;
+        int page = table[kb / page_size];
+        no_page_next = page < 0;
+        if (no_page_next) {
+            if (error_flag && tid == 0) atomicOr(error_flag, 2);    // a visible key has no page
+            page = 0;
+        }
+        const int in_page = kb % page_size;
+        const __bf16* kbase = k_cache + ((int64_t)page * page_size + in_page) * width;
+        const __bf16* vbase = v_cache + ((int64_t)page * tiles_per_page + in_page / LAT_TILE) * rank * LAT_TILE;
+#pragma unroll
+        for (int i = 0; i < KP; ++i) {
+            const int p = tid + 256 * i;
+            if (p < k_pieces) kreg[i] = *reinterpret_cast<const lat_bf16x8*>(kbase + (int64_t)p * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < VP; ++i) {
+            const int p = tid + 256 * i;
+            if (p < v_pieces) vreg[i] = *reinterpret_cast<const lat_bf16x8*>(vbase + (int64_t)p * 8);
+        }
+    };
+    auto put = [&]() __attribute__((always_inline)) {
+        const int per_key = width / 8;
+#pragma unroll
+        for (int i = 0; i < KP; ++i) {
+            const int p = tid + 256 * i;
+            if (p < k_pieces) *reinterpret_cast<lat_bf16x8*>(&k_s[(p / per_key) * KSTR + (p % per_key) * 8]) = kreg[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VP; ++i) {
+            const int p = tid + 256 * i;
+            if (p < v_pieces) {
+                // (rows of 36 elements: two 8-byte stores)
+                lat_bf16x4 lo, hi;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) lo[e] = vreg[i][e], hi[e] = vreg[i][4 + e];
+                __bf16* dst = &v_s[(p / 4) * VSTR + (p % 4) * 8];
+                *reinterpret_cast<lat_bf16x4*>(dst) = lo;
+                *reinterpret_cast<lat_bf16x4*>(dst + 4) = hi;
+            }
+        }
+    };
+    ask(0);
+    for (int tile = 0; tile < tiles; ++tile) {
+        const int kb = tile * LAT_TILE;
+        put();
+        no_page = no_page_next;
+        __syncthreads();
+        if (tile + 1 < tiles) ask(tile + 1);
+        if (kb <= pos) {                                    // (the same for the whole wave)
+            lat_f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < KS; ++c) {
+                if (c < steps) {
+                    lat_bf16x8 ka, kc;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) ka[e] = kc[e] = (__bf16)0.f;
+                    if (32 * c + 8 * g < width) {
+                        ka = *reinterpret_cast<const lat_bf16x8*>(&k_s[col * KSTR + 32 * c + 8 * g]);
+                        kc = *reinterpret_cast<const lat_bf16x8*>(&k_s[(16 + col) * KSTR + 32 * c + 8 * g]);
+                    }
+                    sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[c], sa, 0, 0, 0);
+                    sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kc, qf[c], sb, 0, 0, 0);
+                }
+            }
+            float s[8];
+            float m_new = m_run;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int key = kb + (i < 4 ? 4 * g + i : 16 + 4 * g + i - 4);
+                const float raw = (i < 4 ? sa[i] : sb[i - 4]) * scale;
+                s[i] = key <= pos && !no_page ? raw : -INFINITY;
+                m_new = fmaxf(m_new, s[i]);
+            }
+            m_new = nva_max_over_rows(m_new);
+            const float m_use = fmaxf(m_new, -1e30f);
+            lat_bf16x8 pf;
+            float psum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const __bf16 p = (__bf16)__builtin_amdgcn_exp2f((s[i] - m_use) * log2e);
+                pf[i] = p;
+                psum += (float)p;
+            }
+            psum = nva_sum_over_rows(psum);
+            const float alpha = __builtin_amdgcn_exp2f((fmaxf(m_run, -1e30f) - m_use) * log2e);
+            l_run = l_run * alpha + psum;
+            m_run = m_new;
+            const bool whole = kb + LAT_TILE - 1 <= pos && !no_page;
+#pragma unroll
+            for (int b = 0; b < CB; ++b) {
+                if (b < blocks) {
+                    const lat_bf16x4 lo = *reinterpret_cast<const lat_bf16x4*>(&v_s[(16 * b + col) * VSTR + 4 * g]);
+                    const lat_bf16x4 hi = *reinterpret_cast<const lat_bf16x4*>(&v_s[(16 * b + col) * VSTR + 16 + 4 * g]);
+                    lat_bf16x8 vf;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) vf[e] = lo[e], vf[4 + e] = hi[e];
+                    if (!whole) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (no_page || kb + (e < 4 ? 4 * g + e : 16 + 4 * g + e - 4) > pos) vf[e] = (__bf16)0.f;
+                    }
+                    lat_f32x4 a = acc[b];
+                    a[0] *= alpha; a[1] *= alpha; a[2] *= alpha; a[3] *= alpha;
+                    acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, a, 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();                                    // all have read the tile: the next may be stored
+    }
+    if (!head_ok || !token_ok) return;
+    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+    __bf16* orow = out + t * out_stride + (int64_t)head * rank;
+#pragma unroll
+    for (int b = 0; b < CB; ++b)
+        if (b < blocks) {
+            lat_bf16x4 v;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = (__bf16)(acc[b][i] * inv);
+            *reinterpret_cast<lat_bf16x4*>(orow + 16 * b + 4 * g) = v;
+        }
+}
+
 // One wave per (token, head, 128 channels): the shares' results joined, in the order of the shares.
 __global__ void __launch_bounds__(NVA_WAVE)
 latent_attn_merge_kernel(const float* __restrict__ part, int shares, __bf16* __restrict__ out, int64_t out_stride,
@@ -466,6 +647,50 @@ NVA_EXPORT int nva_latent_attention_bf16(const void* q2, int64_t q_stride, void*
                            dim3(NVA_WAVE), 0, stream, part,
                            shares, (__bf16*)out, out_stride, heads, rank);
     return nva_check_launch("latent_attention");
+}
+
+// The portions of prompts of a step: row_tiles is int32 [num_tiles][2] = (request, row tile of 32 queries), requests described
+// by cu_seqlens_q and kv_lens as for the other prefill kernels; q2 and out hold all the step's tokens.  Takes what
+// nva_latent_attention takes, and returns 1 for what it does not.
+NVA_EXPORT int nva_latent_attention_prefill_bf16(const void* q2, int64_t q_stride, void* out, int64_t out_stride,
+                                                 const void* k_cache, const void* v_cache, const int32_t* block_tables,
+                                                 int table_stride, const int32_t* cu_seqlens_q, const int32_t* kv_lens,
+                                                 const int32_t* row_tiles, int64_t num_tiles, int heads, int rank, int rot,
+                                                 int page_size, float scale, const float* sinks, int32_t* error_flag,
+                                                 hipStream_t stream) {
+    if (num_tiles == 0) return 0;
+    if (rank % 16 || rank <= 0 || rank > 512 || rot % 8 || rot <= 0 || rot > LAT_MAX_ROT || page_size % LAT_TILE || page_size <= 0) {
+        nva_fail("latent_attention_prefill: sizes it does not take (%d, %d, %d)", rank, rot, page_size);
+        return 1;
+    }
+    if (!row_tiles || num_tiles < 0 || num_tiles * 8 > 0x7fffffff || heads <= 0 || table_stride <= 0 || !(scale > 0.f))
+        return nva_fail("latent_attention_prefill: bad sizes tiles=%lld heads=%d", (long long)num_tiles, heads);
+    if (q_stride % 8 || out_stride % 4 || !nva_aligned(q2, 16) || !nva_aligned(out, 8) || !nva_aligned(k_cache, 16) ||
+        !nva_aligned(v_cache, 16)) {
+        nva_fail("latent_attention_prefill: rows that are not aligned for vector access");
+        return 1;
+    }
+    const size_t lds = ((size_t)LAT_TILE * (rank + rot + 8) + (size_t)rank * (LAT_TILE + 4)) * sizeof(__bf16);
+    dim3 grid((unsigned)(num_tiles * 8), 1, (unsigned)((heads + 15) / 16));
+#define LAT_LAUNCH(MC)                                                                                               \
+    do {                                                                                                             \
+        auto kernel = latent_attn_quad_kernel<MC>;                                                                   \
+        static bool raised = false;                                                                                  \
+        if (!raised && lds > 48 * 1024) {                                                                            \
+            if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) != hipSuccess) \
+                return nva_fail("latent_attention_prefill: cannot have %zu bytes of LDS", lds);                      \
+            raised = true;                                                                                           \
+        }                                                                                                            \
+        hipLaunchKernelGGL(kernel, grid, dim3(4 * NVA_WAVE), lds, stream, (const __bf16*)q2, q_stride, (__bf16*)out,     \
+                           out_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, block_tables, table_stride,      \
+                           cu_seqlens_q, kv_lens, row_tiles, heads, rank, rot, page_size, scale, sinks, error_flag);    \
+    } while (0)
+    if (rank <= 128) LAT_LAUNCH(128);
+    else if (rank <= 256) LAT_LAUNCH(256);
+    else if (rank <= 384) LAT_LAUNCH(384);
+    else LAT_LAUNCH(512);
+#undef LAT_LAUNCH
+    return nva_check_launch("latent_attention_prefill");
 }
 #endif
 

@@ -1472,15 +1472,26 @@ class HipKernels:
             _i32(batch.token_seq, tokens, "token_seq")
             _i32(batch.positions, tokens, "positions")
             out = torch.empty((tokens, heads * rank), dtype=q2.dtype, device=q2.device)
-            # few tokens with many keys: a token's tiles of 32 keys are shared out, four tiles a share or more, until
-            # about two waves a compute unit run; the number follows from the step's shape alone
-            blocks = (heads + 15) // 16
-            shares = max(1, min(64, ((batch.max_kv_len + 31) // 32) // 4, 512 // (tokens * blocks)))
-            part = torch.empty(tokens * heads * shares * (2 + rank), dtype=torch.float32, device=q2.device) if shares > 1 else None
-            library.call("latent", "bf16", "nva_latent_attention", _p(q2), c_i64(qs), _p(out), c_i64(out.shape[1]), _p(part),
-                         c_i32(shares), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.token_seq),
-                         _p(batch.positions), c_i64(tokens), c_i32(heads), c_i32(rank), c_i32(rot), c_i32(page_size),
-                         c_f32(scale), _p(sinks), _p(self.fault_flag), self._stream())
+            if any(n != 1 for n in batch.q_lens[:batch.num_decode]):
+                raise KernelError("latent attention: the first num_decode requests of a batch must bring one token each")
+            single = batch.num_decode if tokens > batch.num_decode else tokens
+            if single < tokens:
+                # portions of prompts: four tokens in a row to a workgroup, the tiles of keys through LDS once for all four
+                tiles = self._prefill_tiles(batch, q2.device)
+                library.call("latent", "bf16", "nva_latent_attention_prefill", _p(q2), c_i64(qs), _p(out), c_i64(out.shape[1]),
+                             _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.cu_seqlens_q),
+                             _p(batch.kv_lens), _p(tiles), c_i64(tiles.shape[0]), c_i32(heads), c_i32(rank), c_i32(rot),
+                             c_i32(page_size), c_f32(scale), _p(sinks), _p(self.fault_flag), self._stream())
+            if single > 0:
+                # few tokens with many keys: a token's tiles of 32 keys are shared out, four tiles a share or more, until
+                # about two waves a compute unit run; the number follows from the step's shape alone
+                blocks = (heads + 15) // 16
+                shares = max(1, min(64, ((batch.max_kv_len + 31) // 32) // 4, 512 // (single * blocks)))
+                part = torch.empty(single * heads * shares * (2 + rank), dtype=torch.float32, device=q2.device) if shares > 1 else None
+                library.call("latent", "bf16", "nva_latent_attention", _p(q2), c_i64(qs), _p(out), c_i64(out.shape[1]), _p(part),
+                             c_i32(shares), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.token_seq),
+                             _p(batch.positions), c_i64(single), c_i32(heads), c_i32(rank), c_i32(rot), c_i32(page_size),
+                             c_f32(scale), _p(sinks), _p(self.fault_flag), self._stream())
             return out
         return self.paged_attention(q2, heads, 1, rank + rot, k_cache, v_cache, batch, group, scale, None, v_head_dim=rank,
                                     sinks=sinks)
