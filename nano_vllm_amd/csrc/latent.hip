@@ -390,37 +390,39 @@ latent_attn_kernel(const __bf16* __restrict__ q2, int64_t q_stride, __bf16* __re
         }
 }
 
-// The same attention for portions of prompts: a workgroup of four waves takes four tokens in a row of one request (a
-// quarter of an eighth of a row tile of 32 queries; tiles as for the other prefill kernels, most keys first), a wave one
-// token.  The tiles of keys and of transposed values, which the four tokens share, go through LDS once for all of them:
+// The same attention for portions of prompts: a workgroup of WAVES waves (eight, or four where a latent of more than
+// 384 channels leaves a SIMD's registers to one wave) takes as many tokens in a row of one request (a part of a row tile
+// of 32 queries; tiles as for the other prefill kernels, most keys first), a wave one token.  The tiles of keys and of
+// transposed values, which the tokens share, go through LDS once for all of them:
 // the next tile is asked for (into registers) before the products of the tile at hand and stored after them.  The
 // arithmetic of a token is that of latent_attn_kernel with one share, operation for operation.
-template <int MAXC>
-__global__ void __launch_bounds__(4 * NVA_WAVE)
+template <int MAXC, int WAVES>
+__global__ void __launch_bounds__(WAVES * NVA_WAVE)
 latent_attn_quad_kernel(const __bf16* __restrict__ q2, int64_t q_stride, __bf16* __restrict__ out, int64_t out_stride,
                         const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
                         const int32_t* __restrict__ block_tables, int table_stride, const int32_t* __restrict__ cu_seqlens_q,
                         const int32_t* __restrict__ kv_lens, const int32_t* __restrict__ row_tiles, int heads, int rank, int rot,
                         int page_size, float scale, const float* __restrict__ sinks, int32_t* error_flag) {
     constexpr int KS = (MAXC + LAT_MAX_ROT) / 32, CB = MAXC / 16;
-    constexpr int KP = (MAXC + LAT_MAX_ROT) / 64, VP = MAXC / 64;       // 16-byte pieces of a tile a thread moves, at most
+    constexpr int THREADS = WAVES * NVA_WAVE, PER_TILE = 32 / WAVES;   // tokens of a workgroup: WAVES; workgroups of a row tile
+    constexpr int KP = (4 * (MAXC + LAT_MAX_ROT) + THREADS - 1) / THREADS, VP = (4 * MAXC + THREADS - 1) / THREADS;   // 16-byte pieces of a tile a thread moves, at most
     extern __shared__ __attribute__((aligned(16))) __bf16 lat_s[];
     const int width = rank + rot, KSTR = width + 8, VSTR = LAT_TILE + 4;
     __bf16* const k_s = lat_s;                          // [32 keys][KSTR]
     __bf16* const v_s = lat_s + LAT_TILE * KSTR;        // [rank channels][VSTR]
-    const int ti = blockIdx.x / 8, quad = blockIdx.x % 8;
+    const int ti = blockIdx.x / PER_TILE, quad = blockIdx.x % PER_TILE;
     const int seq = row_tiles[2 * ti], row_tile = row_tiles[2 * ti + 1];
     const int q_begin = cu_seqlens_q[seq];
     const int q_len = cu_seqlens_q[seq + 1] - q_begin;
     const int start = kv_lens[seq] - q_len;             // position of the request's first query of this step
-    const int row0 = row_tile * 32 + quad * 4;
+    const int row0 = row_tile * 32 + quad * WAVES;
     if (row0 >= q_len) return;                          // (the whole workgroup)
     const int tid = threadIdx.x, wave = tid / NVA_WAVE, lane = tid % NVA_WAVE, col = lane & 15, g = lane >> 4;
     const int row = row0 + wave;
     const bool token_ok = row < q_len;
     const int pos = token_ok ? start + row : -1;
     const int64_t t = q_begin + (token_ok ? row : row0);
-    const int tiles = (start + min(row0 + 3, q_len - 1)) / LAT_TILE + 1;
+    const int tiles = (start + min(row0 + WAVES - 1, q_len - 1)) / LAT_TILE + 1;
     const int head = blockIdx.z * 16 + col;
     const bool head_ok = head < heads;
     const int steps = (width + 31) / 32, blocks = rank / 16;
@@ -458,12 +460,12 @@ latent_attn_quad_kernel(const __bf16* __restrict__ q2, int64_t q_stride, __bf16*
         const __bf16* vbase = v_cache + ((int64_t)page * tiles_per_page + in_page / LAT_TILE) * rank * LAT_TILE;
 #pragma unroll
         for (int i = 0; i < KP; ++i) {
-            const int p = tid + 256 * i;
+            const int p = tid + THREADS * i;
             if (p < k_pieces) kreg[i] = *reinterpret_cast<const lat_bf16x8*>(kbase + (int64_t)p * 8);
         }
 #pragma unroll
         for (int i = 0; i < VP; ++i) {
-            const int p = tid + 256 * i;
+            const int p = tid + THREADS * i;
             if (p < v_pieces) vreg[i] = *reinterpret_cast<const lat_bf16x8*>(vbase + (int64_t)p * 8);
         }
     };
@@ -471,12 +473,12 @@ latent_attn_quad_kernel(const __bf16* __restrict__ q2, int64_t q_stride, __bf16*
         const int per_key = width / 8;
 #pragma unroll
         for (int i = 0; i < KP; ++i) {
-            const int p = tid + 256 * i;
+            const int p = tid + THREADS * i;
             if (p < k_pieces) *reinterpret_cast<lat_bf16x8*>(&k_s[(p / per_key) * KSTR + (p % per_key) * 8]) = kreg[i];
         }
 #pragma unroll
         for (int i = 0; i < VP; ++i) {
-            const int p = tid + 256 * i;
+            const int p = tid + THREADS * i;
             if (p < v_pieces) {
                 // (rows of 36 elements: two 8-byte stores)
                 lat_bf16x4 lo, hi;
@@ -671,24 +673,25 @@ NVA_EXPORT int nva_latent_attention_prefill_bf16(const void* q2, int64_t q_strid
         return 1;
     }
     const size_t lds = ((size_t)LAT_TILE * (rank + rot + 8) + (size_t)rank * (LAT_TILE + 4)) * sizeof(__bf16);
-    dim3 grid((unsigned)(num_tiles * 8), 1, (unsigned)((heads + 15) / 16));
-#define LAT_LAUNCH(MC)                                                                                               \
+    const int waves = rank <= 384 ? 8 : 4;       // tokens of a workgroup (what the registers of a SIMD hold two waves of)
+    dim3 grid((unsigned)(num_tiles * (32 / waves)), 1, (unsigned)((heads + 15) / 16));
+#define LAT_LAUNCH(MC, WV)                                                                                           \
     do {                                                                                                             \
-        auto kernel = latent_attn_quad_kernel<MC>;                                                                   \
+        auto kernel = latent_attn_quad_kernel<MC, WV>;                                                                 \
         static bool raised = false;                                                                                  \
         if (!raised && lds > 48 * 1024) {                                                                            \
             if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) != hipSuccess) \
                 return nva_fail("latent_attention_prefill: cannot have %zu bytes of LDS", lds);                      \
             raised = true;                                                                                           \
         }                                                                                                            \
-        hipLaunchKernelGGL(kernel, grid, dim3(4 * NVA_WAVE), lds, stream, (const __bf16*)q2, q_stride, (__bf16*)out,     \
+        hipLaunchKernelGGL(kernel, grid, dim3(WV * NVA_WAVE), lds, stream, (const __bf16*)q2, q_stride, (__bf16*)out,    \
                            out_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, block_tables, table_stride,      \
                            cu_seqlens_q, kv_lens, row_tiles, heads, rank, rot, page_size, scale, sinks, error_flag);    \
     } while (0)
-    if (rank <= 128) LAT_LAUNCH(128);
-    else if (rank <= 256) LAT_LAUNCH(256);
-    else if (rank <= 384) LAT_LAUNCH(384);
-    else LAT_LAUNCH(512);
+    if (rank <= 128) LAT_LAUNCH(128, 8);
+    else if (rank <= 256) LAT_LAUNCH(256, 8);
+    else if (rank <= 384) LAT_LAUNCH(384, 8);
+    else LAT_LAUNCH(512, 4);
 #undef LAT_LAUNCH
     return nva_check_launch("latent_attention_prefill");
 }
