@@ -360,7 +360,7 @@ def _run_latent(k, dev, dtype, batch, all_slots, kc, vc, rows, w, H_, D, R, DV, 
     (2, 64, 16, 32, 176, 64, [100], [37]),                    # key rows of more than 128 entries
     (2, 16, 32, 16, 96, 64, [1, 200], [1, 150]),              # key rows of exactly 128, the first token of a sequence
     (20, 32, 64, 32, 384, 64, [1500, 33, 700], [1, 1, 40]),   # more heads than a tile of columns, shares of a token's keys
-    (4, 32, 16, 32, 96, 32, [1000, 2], [1, 1]),               # a rotated part that ends inside a step of 32 channels
+    (5, 24, 24, 40, 80, 32, [1000, 2], [1, 1]),               # a key row that ends inside a step of 32 channels
 ])
 def test_attention_through_a_latent(backend, dtype, H_, D, R, DV, C, page, lens, q_lens):
     k, dev = _kernels(backend, dtype)
